@@ -1,0 +1,67 @@
+"""Host logic of the step function, on the CPU with plain kernels, against the plain implementation."""
+import pytest
+import torch
+
+from .cpu_engine import load_cpu_model
+from .plain import gemma2_plain as plain
+from .tiny import CONFIGS, make_folder, random_tokens, rel_l2
+
+
+@pytest.fixture(scope="module", params=["A", "B", "C"])
+def setup(request, tmp_path_factory):
+    folder = make_folder(tmp_path_factory.mktemp("m"), request.param)
+    model, cfg = load_cpu_model(folder)
+    pcfg, pw = plain.read_folder(folder)
+    return model, cfg, pcfg, pw
+
+
+def test_whole_prompt_equals_plain(setup):
+    model, cfg, pcfg, pw = setup
+    toks = random_tokens(45, cfg.vocab_size, 3)
+    cache = model.new_cache(max_tokens=256)
+    s = cache.acquire()
+    got = model.step(cache, [s], toks, counts=[len(toks)], want=list(range(len(toks))))
+    ref = plain.forward(pcfg, pw, toks)
+    assert rel_l2(got, ref) < 2e-5
+    cache.release(s)
+
+
+@pytest.mark.parametrize("page_size", [16, 64])
+def test_token_by_token_equals_whole(setup, page_size):
+    model, cfg, pcfg, pw = setup
+    toks = random_tokens(40, cfg.vocab_size, 4)
+    ref = plain.forward(pcfg, pw, toks)
+    cache = model.new_cache(max_tokens=256, page_size=page_size)     # 16: the window's ring wraps
+    s = cache.acquire()
+    rows = [model.step(cache, [s], toks[:8], counts=[8], want=list(range(8)))]
+    for t in toks[8:]:
+        rows.append(model.step(cache, [s], [t]))
+    got = torch.cat(rows)
+    assert rel_l2(got, ref) < 2e-5
+
+
+def test_unequal_batches_and_slot_reuse(setup):
+    model, cfg, pcfg, pw = setup
+    cache = model.new_cache(max_tokens=64 * 3, max_slots=3, page_size=16)
+    for batch, lens in enumerate([(5, 11, 17), (1, 9, 40), (23, 2, 3)]):
+        seqs = [random_tokens(n + 6, cfg.vocab_size, 100 * batch + i) for i, n in enumerate(lens)]
+        extra = [6, 3, 1]                        # decoded tokens per sequence: the shorter ones end earlier
+        slots = [cache.acquire() for _ in lens]
+        flat = [t for s, n in zip(seqs, lens) for t in s[:n]]
+        got = {i: [] for i in range(3)}
+        out = model.step(cache, slots, flat, counts=list(lens))
+        for i in range(3):
+            got[i].append(out[i])
+        for step in range(max(extra)):
+            live = [i for i in range(3) if step < extra[i]]
+            out = model.step(cache, [slots[i] for i in live], [seqs[i][lens[i] + step] for i in live])
+            for j, i in enumerate(live):
+                got[i].append(out[j])
+            for i in range(3):
+                if step + 1 == extra[i]:
+                    cache.release(slots[i])
+        for i in range(3):
+            n = lens[i] + extra[i]
+            ref = plain.forward(pcfg, pw, seqs[i][:n])[lens[i] - 1:n]
+            assert rel_l2(torch.stack(got[i]), ref) < 2e-5, (batch, i)
+    assert cache.live_slots() == []

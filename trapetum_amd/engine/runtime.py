@@ -1,0 +1,56 @@
+"""Where and how a model runs: device, dtype, and the kernels.
+
+dtype "bfloat16": bf16 weights, activations and cache, fp32 residual stream,
+statistics, softmax and logits (the reference's fp16/fp32 split, runtime/src/
+lib.rs:4483-4516, with bf16 in fp16's place).  dtype "float32": every tensor
+and every operation in fp32, no reduced-precision matrix mode.
+"""
+import torch
+
+_DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32}
+
+
+def parse_dtype(name):
+    if isinstance(name, torch.dtype):
+        if name not in (torch.bfloat16, torch.float32):
+            raise ValueError(f"dtype {name} is not supported (bfloat16 or float32)")
+        return name
+    if name not in _DTYPES:
+        raise ValueError(f"dtype '{name}' is not supported (bfloat16 or float32)")
+    return _DTYPES[name]
+
+
+class Runtime:
+    """`ops` is the kernel library; by default the HIP one, which refuses to load without a GPU."""
+
+    def __init__(self, dtype="bfloat16", device="cuda:0", ops=None):
+        self.dtype = parse_dtype(dtype)
+        self.device = torch.device(device)
+        if ops is None:
+            from .. import kernels
+            ops = kernels.load(self.device)
+        self.ops = ops
+        self._staging = []
+        self._next = 0
+
+    def upload_i32(self, array):
+        """Host int32 numpy array -> device tensor (asynchronous from pinned memory on a GPU)."""
+        t = torch.from_numpy(array)
+        if self.device.type != "cuda":
+            return t.clone()
+        n = t.numel()
+        if not self._staging:
+            self._staging = [[torch.empty(4096, dtype=torch.int32, pin_memory=True), None] for _ in range(8)]
+        slot = self._staging[self._next]
+        self._next = (self._next + 1) % len(self._staging)
+        if slot[1] is not None:
+            slot[1].synchronize()
+        if slot[0].numel() < n:
+            slot[0] = torch.empty(max(n, 2 * slot[0].numel()), dtype=torch.int32, pin_memory=True)
+        slot[0][:n].copy_(t.reshape(-1))
+        out = torch.empty(n, dtype=torch.int32, device=self.device)
+        out.copy_(slot[0][:n], non_blocking=True)
+        ev = torch.cuda.Event()
+        ev.record()
+        slot[1] = ev
+        return out.reshape(array.shape)

@@ -1,0 +1,80 @@
+"""Grouped-query attention over the cache, with optional score cap and window.
+
+In the reference's order (runtime/src/lib.rs:4483-4496): q, k, v projections,
+RoPE on q and k, append k (rotated) and v to the cache, attention, output
+projection.  Scores: (q . k) * query_scale, then cap * tanh(s / cap) when a cap is
+set, softmax in fp32 over the visible keys, weighted sum of v; query head h reads
+kv head h // (heads / kv_heads) (runtime/cuda/codebook_gemv.cu:240-270).  The
+reference fixes the scale to rsqrt(head_dim) (cu:249) and has no window
+(lib.rs:4455); both are parameters here: the query at position p sees keys
+t <= p, and with a window W only those with p - t < W.
+
+The three projections are one product over the concatenated weight.  A run that
+reads another run's cache projects and rotates its queries only.
+"""
+from ..cache.store import KVSpec
+from ..models.spec import TensorSpec
+from ..registry import build_part, register_part
+from .base import Mixer
+
+
+class Attention(Mixer):
+    def __init__(self, hidden_size, num_heads, num_kv_heads, head_dim, query_scale,
+                 softcap=None, window=None, position=("none", {})):
+        if num_heads % num_kv_heads:
+            raise ValueError(f"{num_heads} query heads are no multiple of {num_kv_heads} kv heads")
+        self.hidden_size = hidden_size
+        self.num_heads = num_heads
+        self.num_kv_heads = num_kv_heads
+        self.head_dim = head_dim
+        self.query_scale = float(query_scale)
+        self.softcap = float(softcap) if softcap else 0.0
+        self.window = int(window) if window else 0
+        self.position = build_part("position", position)
+        if self.position.rotary_dim > head_dim:
+            raise ValueError(f"rotary_dim {self.position.rotary_dim} exceeds head_dim {head_dim}")
+
+    def tensor_specs(self):
+        d, q, kv = self.hidden_size, self.num_heads * self.head_dim, self.num_kv_heads * self.head_dim
+        return {"q_proj.weight": TensorSpec((q, d)), "k_proj.weight": TensorSpec((kv, d)),
+                "v_proj.weight": TensorSpec((kv, d)), "o_proj.weight": TensorSpec((d, q))}
+
+    def cache_spec(self):
+        return KVSpec(self.num_kv_heads, self.head_dim, self.window or None)
+
+    def bind(self, tensors, rt):
+        import torch
+        self.rt = rt
+        self.w_qkv = torch.cat([tensors["q_proj.weight"], tensors["k_proj.weight"],
+                                tensors["v_proj.weight"]], dim=0).contiguous()
+        self.w_o = tensors["o_proj.weight"]
+        self.inv_freq = self.position.inv_freq(rt.device)
+
+    def forward(self, ctx, x, site):
+        ops = ctx.ops
+        H, KV, hd = self.num_heads, self.num_kv_heads, self.head_dim
+        Q, KVD = H * hd, KV * hd
+        owns_cache = ctx.cache_owner == ctx.entry
+        if owns_cache:
+            qkv = ops.linear(x, self.w_qkv, ctx.dtype)
+            q, k, v = qkv[:, :Q], qkv[:, Q:Q + KVD], qkv[:, Q + KVD:]
+        else:
+            q, k, v = ops.linear(x, self.w_qkv[:Q], ctx.dtype), None, None
+        table = ctx.page_table(site.group_index)
+        rows_cap = site.rows_cap or 0
+        ops.rope_kv_write(q, k, v, H, KV, hd, self.inv_freq, self.position.rotary_dim,
+                          ctx.row_seq, ctx.row_pos, ctx.new_len, table, site.k, site.v, rows_cap)
+        if ctx.mode == "prefill":
+            if owns_cache:
+                ctx.offer_step_kv(k, v)
+            else:
+                k, v = ctx.step_kv_of(ctx.cache_owner)
+            out = ops.attention_prefill(q, k, v, H, KV, hd, ctx.cu_rows, ctx.max_count,
+                                        self.query_scale, self.softcap, self.window, ctx.dtype)
+        else:
+            out = ops.attention_decode(q, H, KV, hd, ctx.new_len, table, site.k, site.v, rows_cap,
+                                       self.query_scale, self.softcap, self.window, ctx.dtype)
+        return ops.linear(out, self.w_o, ctx.dtype)
+
+
+register_part("mixer", "attention", Attention)

@@ -1,0 +1,81 @@
+"""What every part is: sizes and constants as constructor arguments, tensors under local names.
+
+A part never learns which model it stands in.  It declares the tensors it needs
+(`tensor_specs`), receives them on the device (`bind`), and runs on the rows of a
+step (`forward`).  Interfaces:
+
+  Norm         forward(ctx, x, out_dtype) -> rows;  `gain` is the fp32 vector the
+               norm multiplies by, so that blocks can fuse a norm into a neighbour.
+  Position     `rotary_dim` and `inv_freq(device)`: the rotation table a mixer applies
+               to queries and keys before the cache write.
+  Mixer        cache_spec() -> KVSpec | StateSpec | None;
+               forward(ctx, x, site) -> rows [M, hidden], x being the normed rows.
+  FeedForward  forward(ctx, x) -> rows [M, hidden].
+  Block        sites() -> names of its norms;  forward(ctx, stream) -> stream, the
+               residual stream being fp32 [M, hidden].
+  Embedding    forward(ctx, tokens) -> fp32 stream;  Head  forward(ctx, rows) -> fp32 logits.
+
+`ctx` is the step's StepContext: batch geometry on the device, the kernels
+(`ctx.ops`), the activation dtype (`ctx.dtype`) and the cache.
+"""
+
+
+class Part:
+    def tensor_specs(self):
+        """{local tensor name: TensorSpec}."""
+        return {}
+
+    def bind(self, tensors, rt):
+        """Take the tensors ({local name: device tensor}) and prepare what forward needs."""
+        self.rt = rt
+
+
+class Norm(Part):
+    gain = None
+
+    def forward(self, ctx, x, out_dtype=None):
+        raise NotImplementedError
+
+
+class Position(Part):
+    rotary_dim = 0
+
+    def inv_freq(self, device):
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    def cache_spec(self):
+        return None
+
+    def forward(self, ctx, x, site):
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, ctx, x):
+        raise NotImplementedError
+
+
+class Block(Part):
+    def __init__(self, mixer, feed_forward, make_norm):
+        self.mixer = mixer
+        self.feed_forward = feed_forward
+        self.norms = {name: make_norm() for name in self.norm_sites()}
+
+    @classmethod
+    def norm_sites(cls):
+        return ()
+
+    def forward(self, ctx, stream, site):
+        raise NotImplementedError
+
+
+class Embedding(Part):
+    def forward(self, ctx, tokens):
+        raise NotImplementedError
+
+
+class Head(Part):
+    def forward(self, ctx, rows):
+        raise NotImplementedError
