@@ -102,7 +102,7 @@ def _attend(qrow, keys, vals, scale, softcap):
     return p @ vals
 
 
-def attention_prefill(q, k, v, H, KV, hd, cu_rows, max_count, scale, softcap, window, out_dtype):
+def attention_prefill(q, k, v, H, KV, hd, cu_rows, max_count, scale, softcap, window, out_dtype, row_seq=None, row_pos=None):
     m = q.shape[0]
     out = torch.zeros((m, H * hd), dtype=torch.float32, device=q.device)
     qf, kf, vf = q.float().reshape(m, H, hd), k.float().reshape(m, KV, hd), v.float().reshape(m, KV, hd)
@@ -116,7 +116,7 @@ def attention_prefill(q, k, v, H, KV, hd, cu_rows, max_count, scale, softcap, wi
     return out.to(out_dtype)
 
 
-def attention_decode(q, H, KV, hd, new_len, table, k_pool, v_pool, rows_cap, scale, softcap, window, out_dtype):
+def attention_decode(q, H, KV, hd, new_len, table, k_pool, v_pool, rows_cap, scale, softcap, window, out_dtype, max_keys=None):
     n = q.shape[0]
     page = k_pool.shape[2]
     out = torch.zeros((n, H * hd), dtype=torch.float32, device=q.device)

@@ -1,0 +1,84 @@
+"""The engine on the GPU against the plain implementation: whole, token by token, unequal batches, reused slots."""
+import pytest
+import torch
+
+from .plain import gemma2_plain as plain
+from .tiny import make_folder, random_tokens, rel_l2
+
+pytestmark = pytest.mark.gpu
+TOL = {"float32": 1e-5, "bfloat16": 2e-2}
+
+
+@pytest.fixture(scope="module", params=[("A", "float32"), ("A", "bfloat16"), ("B", "float32"), ("B", "bfloat16"),
+                                        ("C", "float32"), ("C", "bfloat16")], ids=lambda p: f"{p[0]}-{p[1]}")
+def setup(request, tmp_path_factory):
+    from .gpu_engine import load_gpu_model
+    which, dtype = request.param
+    folder = make_folder(tmp_path_factory.mktemp("m"), which)
+    model, cfg = load_gpu_model(folder, dtype)
+    pcfg, pw = plain.read_folder(folder)
+    return model, cfg, pcfg, pw, TOL[dtype]
+
+
+def test_whole_prompt(setup):
+    model, cfg, pcfg, pw, tol = setup
+    toks = random_tokens(90, cfg.vocab_size, 3)
+    cache = model.new_cache(max_tokens=256, page_size=16)
+    s = cache.acquire()
+    got = model.step(cache, [s], toks, counts=[len(toks)], want=list(range(len(toks))))
+    ref = plain.forward(pcfg, pw, toks)
+    assert rel_l2(got, ref) < tol
+    cache.release(s)
+
+
+def test_last_32_one_by_one(setup):
+    model, cfg, pcfg, pw, tol = setup
+    toks = random_tokens(75, cfg.vocab_size, 4)
+    ref = plain.forward(pcfg, pw, toks)
+    cache = model.new_cache(max_tokens=256, page_size=16)
+    s = cache.acquire()
+    n0 = len(toks) - 32
+    rows = [model.step(cache, [s], toks[:n0], counts=[n0], want=list(range(n0)))]
+    for t in toks[n0:]:
+        rows.append(model.step(cache, [s], [t]))
+    got = torch.cat(rows)
+    assert rel_l2(got, ref) < tol
+    for i in range(len(toks)):
+        assert rel_l2(got[i], ref[i]) < 3 * tol, i
+
+
+def test_first_tokens(setup):
+    model, cfg, pcfg, pw, tol = setup
+    toks = random_tokens(6, cfg.vocab_size, 5)
+    ref = plain.forward(pcfg, pw, toks)
+    cache = model.new_cache(max_tokens=128)
+    s = cache.acquire()
+    got = torch.cat([model.step(cache, [s], [t]) for t in toks])
+    assert rel_l2(got, ref) < tol
+
+
+def test_unequal_batches_reused_slots(setup):
+    model, cfg, pcfg, pw, tol = setup
+    cache = model.new_cache(max_tokens=16 * 12, max_slots=3, page_size=16)
+    for batch, lens in enumerate([(5, 11, 17), (1, 9, 40), (23, 2, 3)]):
+        seqs = [random_tokens(n + 6, cfg.vocab_size, 100 * batch + i) for i, n in enumerate(lens)]
+        extra = [6, 3, 1]
+        slots = [cache.acquire() for _ in lens]
+        flat = [t for s, n in zip(seqs, lens) for t in s[:n]]
+        got = {i: [] for i in range(3)}
+        out = model.step(cache, slots, flat, counts=list(lens))
+        for i in range(3):
+            got[i].append(out[i])
+        for step in range(max(extra)):
+            live = [i for i in range(3) if step < extra[i]]
+            out = model.step(cache, [slots[i] for i in live], [seqs[i][lens[i] + step] for i in live])
+            for j, i in enumerate(live):
+                got[i].append(out[j])
+            for i in range(3):
+                if step + 1 == extra[i]:
+                    cache.release(slots[i])
+        for i in range(3):
+            n = lens[i] + extra[i]
+            ref = plain.forward(pcfg, pw, seqs[i][:n])[lens[i] - 1:n]
+            assert rel_l2(torch.stack(got[i]), ref) < tol, (batch, i)
+    assert cache.live_slots() == []

@@ -1,0 +1,266 @@
+"""Each HIP kernel alone against its plain torch reference (tests/ref_ops.py), at sizes other than the engine's."""
+import math
+
+import pytest
+import torch
+
+from . import ref_ops
+from .tiny import rel_l2
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+DT = {"f32": torch.float32, "bf16": torch.bfloat16}
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from trapetum_amd import kernels
+    return kernels.load(torch.device(DEV))
+
+
+def randn(*shape, dtype=torch.float32, seed=0, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+def tol(dtype):
+    return 2e-6 if dtype == torch.float32 else 6e-3
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("m,d,v", [(1, 64, 17), (5, 88, 331), (33, 2304, 1000)])
+def test_embed_rows(ops, dt, m, d, v):
+    table = randn(v, d, dtype=DT[dt])
+    tok = torch.randint(0, v, (m,), dtype=torch.int32, device=DEV)
+    got = ops.embed_rows(tok, table, math.sqrt(d))
+    assert torch.equal(got.cpu(), ref_ops.embed_rows(tok.cpu(), table.cpu(), math.sqrt(d)))
+
+
+@pytest.mark.parametrize("din,dout", [("f32", "f32"), ("f32", "bf16"), ("bf16", "bf16"), ("bf16", "f32")])
+@pytest.mark.parametrize("m,d", [(1, 16), (3, 88), (7, 2304), (2, 5000)])
+def test_rms_norm(ops, din, dout, m, d):
+    x = randn(m, d, dtype=DT[din], seed=1, scale=3.0)
+    gain = 1.0 + randn(d, seed=2, scale=0.3)
+    got = ops.rms_norm(x, gain, 1e-5, DT[dout])
+    ref = ref_ops.rms_norm(x.cpu(), gain.cpu(), 1e-5, DT[dout])
+    assert rel_l2(got, ref) < tol(DT[dout])
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("post,nxt", [(True, True), (True, False), (False, True), (False, False)])
+@pytest.mark.parametrize("m,d", [(1, 64), (5, 88), (4, 3584)])
+def test_add_rms_norm(ops, dt, post, nxt, m, d):
+    stream = randn(m, d, seed=3, scale=2.0)
+    rows = randn(m, d, dtype=DT[dt], seed=4, scale=5.0)
+    gp = (1.0 + randn(d, seed=5, scale=0.2)) if post else None
+    gn = (1.0 + randn(d, seed=6, scale=0.2)) if nxt else None
+    ref_stream = stream.cpu().clone()
+    ref = ref_ops.add_rms_norm(ref_stream, rows.cpu(), gp.cpu() if post else None, 1e-6, gn.cpu() if nxt else None, 1e-4, DT[dt])
+    got = ops.add_rms_norm(stream, rows, gp, 1e-6, gn, 1e-4, DT[dt])
+    assert rel_l2(stream, ref_stream) < 2e-6
+    if nxt:
+        assert rel_l2(got, ref) < tol(DT[dt])
+    else:
+        assert got is None
+
+
+def test_gather_rows(ops):
+    x = randn(9, 88)
+    rows = torch.tensor([8, 0, 3, 3], dtype=torch.int32, device=DEV)
+    assert torch.equal(ops.gather_rows(x, rows).cpu(), x.cpu()[[8, 0, 3, 3]])
+
+
+# ---- matrix products: every kernel, ragged edges -------------------------------------------------------
+LINEAR_SHAPES = [(1, 16, 8), (3, 100, 72), (17, 331, 88), (64, 130, 2304), (5, 2304, 2048), (8, 1000, 9216),
+                 (65, 200, 136), (300, 257, 520)]
+
+
+@pytest.mark.parametrize("algo", [1, 2, 3])
+@pytest.mark.parametrize("m,n,k", LINEAR_SHAPES)
+def test_linear_bf16(ops, algo, m, n, k):
+    if algo == 2 and m > 64:
+        pytest.skip("the skinny kernel takes at most 64 rows")
+    x, w = randn(m, k, dtype=torch.bfloat16, seed=7), randn(n, k, dtype=torch.bfloat16, seed=8, scale=0.05)
+    ops.force_linear = algo
+    try:
+        got_b = ops.linear(x, w, torch.bfloat16)
+        got_f = ops.linear(x, w, torch.float32)
+        got_c = ops.linear(x, w, torch.float32, softcap=3.0)
+    finally:
+        ops.force_linear = 0
+    ref = x.cpu().double() @ w.cpu().double().T
+    assert rel_l2(got_f, ref) < 1e-5
+    assert rel_l2(got_b, ref) < 4e-3
+    assert rel_l2(got_c, 3.0 * torch.tanh(ref / 3.0)) < 1e-5
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 16, 8), (3, 100, 71), (70, 331, 88), (5, 700, 2304)])
+def test_linear_f32(ops, m, n, k):
+    x, w = randn(m, k, seed=9), randn(n, k, seed=10, scale=0.05)
+    got = ops.linear(x, w, torch.float32)
+    ref = x.cpu().double() @ w.cpu().double().T
+    assert rel_l2(got, ref) < 2e-6
+    # the sum's order per element does not depend on the other rows: a row alone gives the same bits
+    alone = ops.linear(x[m - 1:m].contiguous(), w, torch.float32)
+    assert torch.equal(alone[0], got[m - 1])
+
+
+@pytest.mark.parametrize("algo", [1, 2, 3])
+@pytest.mark.parametrize("dt", ["bf16", "f32"])
+@pytest.mark.parametrize("m,inter,k", [(1, 16, 16), (4, 200, 88), (40, 320, 96), (9, 1000, 2304), (150, 72, 136)])
+def test_gated_linear(ops, algo, dt, m, inter, k):
+    if dt == "f32" and algo != 1:
+        pytest.skip("float32 runs on the plain kernel only")
+    if algo == 2 and m > 64:
+        pytest.skip("the skinny kernel takes at most 64 rows")
+    wg, wu = randn(inter, k, dtype=DT[dt], seed=11, scale=0.2), randn(inter, k, dtype=DT[dt], seed=12, scale=0.2)
+    x = randn(m, k, dtype=DT[dt], seed=13)
+    packed = ops.pack_gate_up(wg, wu)
+    assert torch.equal(packed.cpu(), ref_ops.pack_gate_up(wg.cpu(), wu.cpu()))
+    ops.force_linear = algo
+    try:
+        got = ops.gated_linear(x, packed, inter, "gelu_tanh", DT[dt])
+    finally:
+        ops.force_linear = 0
+    g, u = x.cpu().double() @ wg.cpu().double().T, x.cpu().double() @ wu.cpu().double().T
+    ref = torch.nn.functional.gelu(g, approximate="tanh") * u
+    assert rel_l2(got, ref) < (5e-6 if dt == "f32" else 4e-3)
+
+
+# ---- RoPE + cache write, attention over pages --------------------------------------------------------------
+def build_cache_case(dt, H, KV, hd, lens, page, rows_cap, n_pages, seed):
+    """Random q/k/v rows for sequences of the given lengths, pushed through rope_kv_write of the reference."""
+    m = sum(lens)
+    q = randn(m, H * hd, dtype=dt, seed=seed)
+    k = randn(m, KV * hd, dtype=dt, seed=seed + 1)
+    v = randn(m, KV * hd, dtype=dt, seed=seed + 2)
+    row_seq = torch.repeat_interleave(torch.arange(len(lens)), torch.tensor(lens)).to(torch.int32)
+    row_pos = torch.cat([torch.arange(n) for n in lens]).to(torch.int32)
+    new_len = torch.tensor(lens, dtype=torch.int32)
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
+    perm = torch.randperm(n_pages, generator=torch.Generator().manual_seed(seed)).tolist()
+    width = max(-(-(min(n, rows_cap) if rows_cap else n) // page) for n in lens)
+    table = torch.full((len(lens), width), -1, dtype=torch.int32)
+    for i, n in enumerate(lens):
+        need = -(-(min(n, rows_cap) if rows_cap else n) // page)
+        for j in range(need):
+            table[i, j] = perm.pop()
+    inv_freq = (1.0 / (10000.0 ** (torch.arange(0, hd, 2, dtype=torch.float32) / hd)))
+    return dict(q=q, k=k, v=v, row_seq=row_seq, row_pos=row_pos, new_len=new_len, cu=cu, table=table, inv_freq=inv_freq)
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("H,KV,hd,lens,page,rows_cap", [
+    (4, 2, 16, (5, 11, 17), 16, 0), (6, 1, 32, (1, 9, 23, 40), 16, 16), (3, 3, 48, (70, 3), 64, 64),
+    (8, 4, 256, (130,), 64, 0), (2, 2, 80, (33, 50), 16, 32)])
+def test_rope_kv_write(ops, dt, H, KV, hd, lens, page, rows_cap):
+    c = build_cache_case(DT[dt], H, KV, hd, lens, page, rows_cap, 24, 20)
+    pools_ref = [torch.zeros(24, KV, page, hd, dtype=DT[dt]) for _ in range(2)]
+    pools = [p.to(DEV) for p in pools_ref]
+    q_ref, k_ref = c["q"].cpu().clone(), c["k"].cpu().clone()
+    ref_ops.rope_kv_write(q_ref, k_ref, c["v"].cpu(), H, KV, hd, c["inv_freq"], hd, c["row_seq"], c["row_pos"],
+                          c["new_len"], c["table"], pools_ref[0], pools_ref[1], rows_cap)
+    ops.rope_kv_write(c["q"], c["k"], c["v"], H, KV, hd, c["inv_freq"].to(DEV), hd, c["row_seq"].to(DEV),
+                      c["row_pos"].to(DEV), c["new_len"].to(DEV), c["table"].to(DEV), pools[0], pools[1], rows_cap)
+    t = 3e-6 if dt == "f32" else 6e-3
+    assert rel_l2(c["q"], q_ref) < t and rel_l2(c["k"], k_ref) < t
+    assert rel_l2(pools[0], pools_ref[0]) < t
+    assert torch.equal(pools[1].cpu(), pools_ref[1])
+    # rows that no sequence owns stay untouched
+    assert torch.equal((pools[0].cpu() != 0).any(dim=-1), (pools_ref[0] != 0).any(dim=-1))
+
+
+ATTN_CASES = [
+    # H, KV, hd, lens, page, window, rows_cap, cap
+    (4, 2, 16, (5, 11, 17), 16, 8, 16, 50.0),
+    (6, 1, 32, (1, 9, 23, 40), 16, 16, 16, 20.0),
+    (3, 3, 48, (70, 3), 16, 5, 16, 8.0),
+    (8, 4, 256, (130, 64), 64, 0, 0, 50.0),
+    (8, 4, 256, (200,), 64, 100, 128, 0.0),
+    (2, 2, 80, (33, 50), 16, 0, 0, 0.0),
+    (16, 2, 128, (300, 17, 129), 64, 0, 0, 30.0),
+    (32, 1, 64, (90,), 16, 0, 0, 0.0),
+]
+
+
+@pytest.mark.parametrize("plain", [True, False])
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("H,KV,hd,lens,page,window,rows_cap,cap", ATTN_CASES)
+def test_attention_prefill(ops, plain, dt, H, KV, hd, lens, page, window, rows_cap, cap):
+    if dt == "f32" and not plain:
+        pytest.skip("float32 runs on the plain kernel only")
+    c = build_cache_case(DT[dt], H, KV, hd, lens, page, rows_cap, 24, 30)
+    scale = 1.0 / math.sqrt(hd * 0.7)
+    ref = ref_ops.attention_prefill(c["q"].cpu(), c["k"].cpu(), c["v"].cpu(), H, KV, hd, c["cu"], max(lens), scale,
+                                    cap, window, torch.float32)
+    ops.force_plain_attention = plain
+    try:
+        got = ops.attention_prefill(c["q"], c["k"], c["v"], H, KV, hd, c["cu"].to(DEV), max(lens), scale, cap, window,
+                                    DT[dt], row_seq=c["row_seq"].to(DEV), row_pos=c["row_pos"].to(DEV))
+    finally:
+        ops.force_plain_attention = False
+    assert rel_l2(got, ref) < (3e-6 if dt == "f32" else 8e-3)
+
+
+@pytest.mark.parametrize("plain", [True, False])
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("H,KV,hd,lens,page,window,rows_cap,cap", ATTN_CASES)
+def test_attention_decode(ops, plain, dt, H, KV, hd, lens, page, window, rows_cap, cap):
+    if dt == "f32" and not plain:
+        pytest.skip("float32 runs on the plain kernel only")
+    n_pages = 24
+    c = build_cache_case(DT[dt], H, KV, hd, lens, page, rows_cap, n_pages, 40)
+    pools_ref = [torch.zeros(n_pages, KV, page, hd, dtype=DT[dt]) for _ in range(2)]
+    # stale rows of an earlier occupant must not leak: fill the pools with large values first
+    for p in pools_ref:
+        p.fill_(7.0)
+    ref_ops.rope_kv_write(c["q"].cpu().clone(), c["k"].cpu().clone(), c["v"].cpu(), H, KV, hd, None, 0, c["row_seq"],
+                          c["row_pos"], c["new_len"], c["table"], pools_ref[0], pools_ref[1], rows_cap)
+    qlast = torch.stack([c["q"].cpu()[int(c["cu"][i + 1]) - 1] for i in range(len(lens))]).contiguous()
+    scale = 1.0 / math.sqrt(hd * 1.3)
+    ref = ref_ops.attention_decode(qlast, H, KV, hd, c["new_len"], c["table"], pools_ref[0], pools_ref[1], rows_cap, scale,
+                                   cap, window, torch.float32)
+    ops.force_plain_attention = plain
+    try:
+        got = ops.attention_decode(qlast.to(DEV), H, KV, hd, c["new_len"].to(DEV), c["table"].to(DEV),
+                                   pools_ref[0].to(DEV), pools_ref[1].to(DEV), rows_cap, scale, cap, window, DT[dt],
+                                   max_keys=max(lens))
+    finally:
+        ops.force_plain_attention = False
+    assert rel_l2(got, ref) < (3e-6 if dt == "f32" else 8e-3)
+
+
+def test_attention_far_key_stands_out(ops):
+    """One key among hundreds carries the answer: its score is made to dominate, so a kernel that drops
+    or misplaces it (a chunk boundary, a page boundary) returns another value row."""
+    H, KV, hd, n, page = 4, 2, 64, 700, 64
+    for target in (0, 63, 64, 333, 699):
+        c = build_cache_case(torch.bfloat16, H, KV, hd, (n,), page, 0, 16, 50 + target)
+        k = c["k"].cpu().float().reshape(n, KV, hd) * 0.05
+        q = torch.zeros(1, H, hd)
+        q[0, :, :] = k[target, :, :].repeat_interleave(H // KV, dim=0) * 4000.0
+        pools = [torch.zeros(16, KV, page, hd, dtype=torch.bfloat16) for _ in range(2)]
+        kb = k.reshape(n, KV * hd).to(torch.bfloat16)
+        ref_ops.rope_kv_write(torch.zeros(n, H * hd, dtype=torch.bfloat16), kb, c["v"].cpu(), H, KV, hd, None, 0,
+                              c["row_seq"], c["row_pos"], c["new_len"], c["table"], pools[0], pools[1], 0)
+        qb = q.reshape(1, H * hd).to(torch.bfloat16)
+        for plain in (True, False):
+            ops.force_plain_attention = plain
+            try:
+                got = ops.attention_decode(qb.to(DEV), H, KV, hd, c["new_len"].to(DEV), c["table"].to(DEV),
+                                           pools[0].to(DEV), pools[1].to(DEV), 0, 1.0, 0.0, 0, torch.bfloat16, max_keys=n)
+            finally:
+                ops.force_plain_attention = False
+            want = c["v"].cpu().float().reshape(n, KV, hd)[target].repeat_interleave(H // KV, dim=0).reshape(1, H * hd)
+            assert rel_l2(got, want) < 2e-2, (target, plain)
+
+
+def test_argmax_ties_and_nan(ops):
+    z = torch.full((3, 7001), -1.0)
+    z[0, 100] = z[0, 7000] = 5.0               # tie: the smaller index wins (runtime/src/bin/opt_check.rs:37-65)
+    z[1, 7000] = 2.0
+    z[2, 0] = float("nan")
+    z[2, 5] = 0.5
+    assert ops.argmax(z.to(DEV)).tolist() == [100, 7000, 5]
+    big = randn(5, 256000, seed=60)
+    assert ops.argmax(big).tolist() == big.cpu().argmax(dim=-1).tolist()

@@ -1,0 +1,112 @@
+// Plain attention kernel for any dtype, head size up to 256 and any grouping: one wave per (row, query head),
+// keys visited one after the other in position order with a running softmax.
+//
+// It is the float32 path's attention for prefill and decode alike (the same instruction sequence per key in
+// both, so a token's result does not depend on how the prompt was cut), and the bf16 path's fallback for
+// shapes the matrix-core kernels refuse.  Formula and order as the reference's attn_k
+// (runtime/cuda/codebook_gemv.cu:240-270): score = dot * scale, cap * tanh(score / cap), softmax, weighted
+// sum of v, kv head = head / (heads / kv_heads); the scale is an argument (rsqrt(head_dim) there), and a
+// window W hides keys with p - t >= W (none there).
+#include "common.h"
+
+struct AttnSimpleArgs {
+    const void* q; long q_stride;
+    // keys and values of the step itself (prefill): rows of sequence s start at cu_rows[s]
+    const void* k; long k_stride; const void* v; long v_stride;
+    const int* cu_rows; const int* row_seq; const int* row_pos;
+    // keys and values in the paged cache (decode): sequence i is row i, its last position new_len[i] - 1
+    const int* new_len; const int* table; int table_w; const void* k_pool; const void* v_pool; int page; int rows_cap;
+    void* out;
+    int H, KV, hd; float scale, cap; int window; int paged;
+};
+
+template <typename T>
+__global__ void __launch_bounds__(64)
+attn_simple_k(AttnSimpleArgs a) {
+    const int h = blockIdx.y, r = blockIdx.x, lane = threadIdx.x;
+    const int g = h / (a.H / a.KV);
+    int seq, p;
+    if (a.paged) { seq = r; p = a.new_len[r] - 1; }
+    else { seq = a.row_seq[r]; p = a.row_pos[r]; }
+    const int lo = a.window > 0 ? max(0, p - a.window + 1) : 0;
+    const T* q = (const T*)a.q + (size_t)r * a.q_stride + (size_t)h * a.hd;
+    float qv[4], o[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int d = lane + 64 * j;
+        qv[j] = d < a.hd ? ld_f32(q + d) : 0.f;
+        o[j] = 0.f;
+    }
+    float m = -INFINITY, l = 0.f;
+    for (int t = lo; t <= p; t++) {
+        const T *kp, *vp;
+        if (a.paged) {
+            const int row = a.rows_cap > 0 ? t % a.rows_cap : t;
+            const int pg = a.table[(size_t)seq * a.table_w + row / a.page];
+            const size_t off = (((size_t)pg * a.KV + g) * a.page + row % a.page) * a.hd;
+            kp = (const T*)a.k_pool + off;
+            vp = (const T*)a.v_pool + off;
+        } else {
+            const size_t row = (size_t)(a.cu_rows[seq] + t);
+            kp = (const T*)a.k + row * a.k_stride + (size_t)g * a.hd;
+            vp = (const T*)a.v + row * a.v_stride + (size_t)g * a.hd;
+        }
+        float part = 0.f, vv[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int d = lane + 64 * j;
+            const bool ok = d < a.hd;
+            part = fmaf(qv[j], ok ? ld_f32(kp + d) : 0.f, part);
+            vv[j] = ok ? ld_f32(vp + d) : 0.f;
+        }
+        float s = wave_sum(part) * a.scale;
+        if (a.cap > 0.f) s = softcap_f(s, a.cap);
+        const float m_new = fmaxf(m, s);
+        const float alpha = expf(m - m_new), pr = expf(s - m_new);
+        l = l * alpha + pr;
+#pragma unroll
+        for (int j = 0; j < 4; j++) o[j] = o[j] * alpha + pr * vv[j];
+        m = m_new;
+    }
+    T* out = (T*)a.out + ((size_t)r * a.H + h) * a.hd;
+    const float inv = 1.f / l;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int d = lane + 64 * j;
+        if (d < a.hd) st_f32(out + d, o[j] * inv);
+    }
+}
+
+static int launch(const AttnSimpleArgs& a, int dtype, int M, hipStream_t s) {
+    TP_REQUIRE(M > 0 && a.H > 0 && a.KV > 0 && a.hd > 0, "attention: empty shape rows=%d heads=%d kv=%d head_dim=%d", M, a.H, a.KV, a.hd);
+    TP_REQUIRE(a.H % a.KV == 0, "attention: %d query heads are no multiple of %d kv heads", a.H, a.KV);
+    TP_REQUIRE(a.hd <= 256, "attention (plain kernel): head_dim %d exceeds 256", a.hd);
+    TP_REQUIRE(a.H <= 65535, "attention (plain kernel): %d heads exceed one launch (65535)", a.H);
+    dim3 grid(M, a.H);
+    if (dtype == TP_BF16) attn_simple_k<bf16_t><<<grid, 64, 0, s>>>(a);
+    else if (dtype == TP_F32) attn_simple_k<float><<<grid, 64, 0, s>>>(a);
+    else return tp_fail("attention: unknown dtype %d", dtype);
+    return tp_check_launch("attention (plain kernel)");
+}
+
+extern "C" int tp_attn_simple_prefill(const void* q, long q_stride, const void* k, long k_stride, const void* v, long v_stride,
+                                      int dtype, int M, int H, int KV, int hd, const int* cu_rows, const int* row_seq,
+                                      const int* row_pos, float scale, float cap, int window, void* out, void* stream) {
+    AttnSimpleArgs a{};
+    a.q = q; a.q_stride = q_stride; a.k = k; a.k_stride = k_stride; a.v = v; a.v_stride = v_stride;
+    a.cu_rows = cu_rows; a.row_seq = row_seq; a.row_pos = row_pos;
+    a.out = out; a.H = H; a.KV = KV; a.hd = hd; a.scale = scale; a.cap = cap; a.window = window; a.paged = 0;
+    return launch(a, dtype, M, (hipStream_t)stream);
+}
+
+extern "C" int tp_attn_simple_decode(const void* q, long q_stride, int dtype, int n_seq, int H, int KV, int hd,
+                                     const int* new_len, const int* table, int table_w, const void* k_pool,
+                                     const void* v_pool, int page, int rows_cap, float scale, float cap, int window,
+                                     void* out, void* stream) {
+    TP_REQUIRE(page > 0 && table_w > 0, "attention: page size %d, table width %d", page, table_w);
+    AttnSimpleArgs a{};
+    a.q = q; a.q_stride = q_stride; a.new_len = new_len; a.table = table; a.table_w = table_w;
+    a.k_pool = k_pool; a.v_pool = v_pool; a.page = page; a.rows_cap = rows_cap;
+    a.out = out; a.H = H; a.KV = KV; a.hd = hd; a.scale = scale; a.cap = cap; a.window = window; a.paged = 1;
+    return launch(a, dtype, n_seq, (hipStream_t)stream);
+}

@@ -1,0 +1,229 @@
+// Row-wise kernels: embedding, norms fused with the residual add, row gather, RoPE + cache write,
+// gated activation.  One block per row; statistics, angles and sums in fp32.
+#include "common.h"
+#include <string>
+
+// ---- error channel (defined once for the library) ----------------------------------------------
+static thread_local std::string g_error;
+extern "C" const char* tp_last_error() { return g_error.c_str(); }
+int tp_fail(const char* fmt, ...) {
+    char buf[1024];
+    va_list ap; va_start(ap, fmt); vsnprintf(buf, sizeof buf, fmt, ap); va_end(ap);
+    g_error = buf;
+    return 1;
+}
+int tp_check_launch(const char* what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return tp_fail("%s: launch failed: %s", what, hipGetErrorString(e));
+    return 0;
+}
+
+// ---- embedding: out[r] = table[token[r]] * scale (fp32).  Reference: host gather of a pre-scaled fp16
+// row, runtime/src/lib.rs:4555, model/export_gemma.py:59-61. -----------------------------------------
+template <typename T>
+__global__ void embed_rows_k(const int* __restrict__ tokens, const T* __restrict__ table, float scale,
+                             float* __restrict__ out, int D, int V) {
+    const int r = blockIdx.x;
+    int tok = tokens[r];
+    const bool ok = tok >= 0 && tok < V;
+    if (!ok) tok = 0;
+    const T* src = table + (size_t)tok * D;
+    float* dst = out + (size_t)r * D;
+    for (int i = threadIdx.x; i < D; i += blockDim.x) dst[i] = ok ? ld_f32(src + i) * scale : __uint_as_float(0x7fc00000u);
+}
+
+extern "C" int tp_embed_rows(const int* tokens, const void* table, int dtype, float scale, float* out,
+                             int M, int D, int V, void* stream) {
+    TP_REQUIRE(M > 0 && D > 0 && V > 0, "embed_rows: empty shape M=%d D=%d V=%d", M, D, V);
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == TP_BF16) embed_rows_k<bf16_t><<<M, 256, 0, s>>>(tokens, (const bf16_t*)table, scale, out, D, V);
+    else if (dtype == TP_F32) embed_rows_k<float><<<M, 256, 0, s>>>(tokens, (const float*)table, scale, out, D, V);
+    else return tp_fail("embed_rows: unknown dtype %d", dtype);
+    return tp_check_launch("embed_rows");
+}
+
+// ---- RMSNorm: out = x * rsqrt(mean(x^2) + eps) * gain.  runtime/cuda/codebook_gemv.cu:192-202 ---------
+template <typename TI, typename TO>
+__global__ void rms_norm_k(const TI* __restrict__ x, const float* __restrict__ gain, float eps,
+                           TO* __restrict__ out, int D) {
+    __shared__ float red[16];
+    const TI* xr = x + (size_t)blockIdx.x * D;
+    TO* orow = out + (size_t)blockIdx.x * D;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < D; i += blockDim.x) { float v = ld_f32(xr + i); ss += v * v; }
+    ss = block_sum(ss, red);
+    const float scale = rsqrtf(ss / (float)D + eps);
+    for (int i = threadIdx.x; i < D; i += blockDim.x) st_f32(orow + i, (ld_f32(xr + i) * scale) * gain[i]);
+}
+
+extern "C" int tp_rms_norm(const void* x, int in_dtype, const float* gain, float eps, void* out, int out_dtype,
+                           int M, int D, void* stream) {
+    TP_REQUIRE(M > 0 && D > 0, "rms_norm: empty shape M=%d D=%d", M, D);
+    hipStream_t s = (hipStream_t)stream;
+    if (in_dtype == TP_F32 && out_dtype == TP_F32) rms_norm_k<float, float><<<M, 256, 0, s>>>((const float*)x, gain, eps, (float*)out, D);
+    else if (in_dtype == TP_F32 && out_dtype == TP_BF16) rms_norm_k<float, bf16_t><<<M, 256, 0, s>>>((const float*)x, gain, eps, (bf16_t*)out, D);
+    else if (in_dtype == TP_BF16 && out_dtype == TP_F32) rms_norm_k<bf16_t, float><<<M, 256, 0, s>>>((const bf16_t*)x, gain, eps, (float*)out, D);
+    else if (in_dtype == TP_BF16 && out_dtype == TP_BF16) rms_norm_k<bf16_t, bf16_t><<<M, 256, 0, s>>>((const bf16_t*)x, gain, eps, (bf16_t*)out, D);
+    else return tp_fail("rms_norm: unknown dtypes %d -> %d", in_dtype, out_dtype);
+    return tp_check_launch("rms_norm");
+}
+
+// ---- stream += norm_post(rows) (or rows); out = norm_next(stream).  The reference runs rmsnorm, an add in
+// fp32 and the next rmsnorm as three launches: runtime/src/lib.rs:4532-4535, cu:539-542. -----------------
+template <typename T>
+__global__ void add_rms_norm_k(float* __restrict__ stream, const T* __restrict__ rows,
+                               const float* __restrict__ gain_post, float eps_post,
+                               const float* __restrict__ gain_next, float eps_next,
+                               T* __restrict__ out, int D) {
+    __shared__ float red[16];
+    float* sr = stream + (size_t)blockIdx.x * D;
+    const T* ar = rows + (size_t)blockIdx.x * D;
+    float scale_a = 1.f;
+    if (gain_post) {
+        float ss = 0.f;
+        for (int i = threadIdx.x; i < D; i += blockDim.x) { float v = ld_f32(ar + i); ss += v * v; }
+        ss = block_sum(ss, red);
+        scale_a = rsqrtf(ss / (float)D + eps_post);
+    }
+    float ss2 = 0.f;
+    for (int i = threadIdx.x; i < D; i += blockDim.x) {
+        float a = ld_f32(ar + i);
+        if (gain_post) a = (a * scale_a) * gain_post[i];
+        const float v = sr[i] + a;
+        sr[i] = v;
+        ss2 += v * v;
+    }
+    if (!gain_next) return;
+    ss2 = block_sum(ss2, red);
+    const float scale_s = rsqrtf(ss2 / (float)D + eps_next);
+    T* orow = out + (size_t)blockIdx.x * D;
+    for (int i = threadIdx.x; i < D; i += blockDim.x) st_f32(orow + i, (sr[i] * scale_s) * gain_next[i]);   // own writes
+}
+
+extern "C" int tp_add_rms_norm(float* stream, const void* rows, int dtype, const float* gain_post, float eps_post,
+                               const float* gain_next, float eps_next, void* out, int M, int D, void* stream_) {
+    TP_REQUIRE(M > 0 && D > 0, "add_rms_norm: empty shape M=%d D=%d", M, D);
+    TP_REQUIRE(!gain_next || out, "add_rms_norm: a next norm needs an output buffer");
+    hipStream_t s = (hipStream_t)stream_;
+    if (dtype == TP_BF16) add_rms_norm_k<bf16_t><<<M, 256, 0, s>>>(stream, (const bf16_t*)rows, gain_post, eps_post, gain_next, eps_next, (bf16_t*)out, D);
+    else if (dtype == TP_F32) add_rms_norm_k<float><<<M, 256, 0, s>>>(stream, (const float*)rows, gain_post, eps_post, gain_next, eps_next, (float*)out, D);
+    else return tp_fail("add_rms_norm: unknown dtype %d", dtype);
+    return tp_check_launch("add_rms_norm");
+}
+
+// ---- gather rows of the fp32 stream -------------------------------------------------------------------
+__global__ void gather_rows_k(const float* __restrict__ x, const int* __restrict__ rows, float* __restrict__ out, int D, int M) {
+    int r = rows[blockIdx.x];
+    r = r < 0 ? 0 : (r >= M ? M - 1 : r);
+    const float* src = x + (size_t)r * D;
+    float* dst = out + (size_t)blockIdx.x * D;
+    for (int i = threadIdx.x; i < D; i += blockDim.x) dst[i] = src[i];
+}
+
+extern "C" int tp_gather_rows(const float* x, const int* rows, float* out, int n, int D, int M, void* stream) {
+    TP_REQUIRE(n > 0 && D > 0 && M > 0, "gather_rows: empty shape n=%d D=%d M=%d", n, D, M);
+    gather_rows_k<<<n, 256, 0, (hipStream_t)stream>>>(x, rows, out, D, M);
+    return tp_check_launch("gather_rows");
+}
+
+// ---- RoPE on q and k in place, then k and v into the paged cache -----------------------------------------
+// Rotation: pair (d, d + rot/2), angle = pos * inv_freq[d], fp32 cos/sin (runtime/cuda/codebook_gemv.cu:219-230);
+// the cache keeps k after the rotation and v as projected (runtime/src/lib.rs:4487-4490).
+// A sequence's position p lives in row p (or p % rows_cap of a ring), found through its page list.
+template <typename T>
+__global__ void rope_kv_write_k(T* __restrict__ q, long q_stride, T* __restrict__ k, long k_stride,
+                                const T* __restrict__ v, long v_stride, int H, int KV, int hd,
+                                const float* __restrict__ inv_freq, int rot,
+                                const int* __restrict__ row_seq, const int* __restrict__ row_pos,
+                                const int* __restrict__ new_len, const int* __restrict__ table, int table_w,
+                                T* __restrict__ k_pool, T* __restrict__ v_pool, int page, int rows_cap) {
+    const int r = blockIdx.x;
+    const int pos = row_pos[r];
+    const int half = rot / 2;
+    if (half > 0) {
+        T* qr = q + (size_t)r * q_stride;
+        for (int i = threadIdx.x; i < H * half; i += blockDim.x) {
+            const int h = i / half, d = i % half;
+            const float ang = (float)pos * inv_freq[d];
+            const float c = cosf(ang), s = sinf(ang);
+            T* a = qr + h * hd + d;
+            const float x0 = ld_f32(a), x1 = ld_f32(a + half);
+            st_f32(a, x0 * c - x1 * s);
+            st_f32(a + half, x1 * c + x0 * s);
+        }
+    }
+    if (!k) return;
+    T* kr = k + (size_t)r * k_stride;
+    if (half > 0) {
+        for (int i = threadIdx.x; i < KV * half; i += blockDim.x) {
+            const int h = i / half, d = i % half;
+            const float ang = (float)pos * inv_freq[d];
+            const float c = cosf(ang), s = sinf(ang);
+            T* a = kr + h * hd + d;
+            const float x0 = ld_f32(a), x1 = ld_f32(a + half);
+            st_f32(a, x0 * c - x1 * s);
+            st_f32(a + half, x1 * c + x0 * s);
+        }
+    }
+    const int seq = row_seq[r];
+    int row = pos;
+    if (rows_cap > 0) {
+        if (pos + rows_cap < new_len[seq]) return;      // a later row of this step takes the same ring row
+        row = pos % rows_cap;
+    }
+    const int pg = table[(size_t)seq * table_w + row / page];
+    if (pg < 0) return;
+    __syncthreads();                                      // the rotated k of this row is read back below
+    const T* vr = v + (size_t)r * v_stride;
+    const int in_page = row % page;
+    for (int i = threadIdx.x; i < KV * hd; i += blockDim.x) {
+        const int h = i / hd, d = i % hd;
+        const size_t dst = (((size_t)pg * KV + h) * page + in_page) * hd + d;
+        k_pool[dst] = kr[i];
+        v_pool[dst] = vr[i];
+    }
+}
+
+extern "C" int tp_rope_kv_write(void* q, long q_stride, void* k, long k_stride, const void* v, long v_stride,
+                                int dtype, int M, int H, int KV, int hd, const float* inv_freq, int rot,
+                                const int* row_seq, const int* row_pos, const int* new_len,
+                                const int* table, int table_w, void* k_pool, void* v_pool,
+                                int page, int rows_cap, void* stream) {
+    TP_REQUIRE(M > 0 && H > 0 && hd > 0, "rope_kv_write: empty shape M=%d H=%d hd=%d", M, H, hd);
+    TP_REQUIRE(rot >= 0 && rot <= hd && rot % 2 == 0, "rope_kv_write: rotary_dim %d must be even and at most head_dim %d", rot, hd);
+    TP_REQUIRE(rot == 0 || inv_freq, "rope_kv_write: a rotation needs its frequency table");
+    TP_REQUIRE(!k || (v && k_pool && v_pool && table && KV > 0 && page > 0 && table_w > 0),
+               "rope_kv_write: keys without values, cache pools or page table");
+    TP_REQUIRE(rows_cap >= 0 && (rows_cap == 0 || rows_cap % page == 0), "rope_kv_write: ring of %d rows is no multiple of the page size %d", rows_cap, page);
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == TP_BF16)
+        rope_kv_write_k<bf16_t><<<M, 256, 0, s>>>((bf16_t*)q, q_stride, (bf16_t*)k, k_stride, (const bf16_t*)v, v_stride, H, KV, hd,
+            inv_freq, rot, row_seq, row_pos, new_len, table, table_w, (bf16_t*)k_pool, (bf16_t*)v_pool, page, rows_cap);
+    else if (dtype == TP_F32)
+        rope_kv_write_k<float><<<M, 256, 0, s>>>((float*)q, q_stride, (float*)k, k_stride, (const float*)v, v_stride, H, KV, hd,
+            inv_freq, rot, row_seq, row_pos, new_len, table, table_w, (float*)k_pool, (float*)v_pool, page, rows_cap);
+    else return tp_fail("rope_kv_write: unknown dtype %d", dtype);
+    return tp_check_launch("rope_kv_write");
+}
+
+// ---- gated activation on a packed gate/up product: y [M, 2*Ip] fp32 with 16 gate columns, then the 16 up
+// columns of the same units, alternating.  out[m, i] = gelu_tanh(g) * u (runtime/cuda/codebook_gemv.cu:531-537).
+template <typename T>
+__global__ void gated_act_k(const float* __restrict__ y, T* __restrict__ out, int I, int Ip2) {
+    const float* yr = y + (size_t)blockIdx.x * Ip2;
+    T* orow = out + (size_t)blockIdx.x * I;
+    for (int i = threadIdx.x; i < I; i += blockDim.x) {
+        const int base = (i >> 4) * 32 + (i & 15);
+        st_f32(orow + i, gelu_tanh_f(yr[base]) * yr[base + 16]);
+    }
+}
+
+extern "C" int tp_gated_act(const float* y, void* out, int dtype, int M, int I, void* stream) {
+    TP_REQUIRE(M > 0 && I > 0, "gated_act: empty shape M=%d I=%d", M, I);
+    const int Ip2 = 2 * ((I + 15) / 16) * 16;
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == TP_BF16) gated_act_k<bf16_t><<<M, 256, 0, s>>>(y, (bf16_t*)out, I, Ip2);
+    else if (dtype == TP_F32) gated_act_k<float><<<M, 256, 0, s>>>(y, (float*)out, I, Ip2);
+    else return tp_fail("gated_act: unknown dtype %d", dtype);
+    return tp_check_launch("gated_act");
+}

@@ -1,0 +1,25 @@
+// Matrix products of the kernel library: Y[M,N] = X[M,K] . W[N,K]^T with fp32 accumulation.
+// W is a checkpoint matrix as stored ([out, in], row-major), X the step's rows.
+#pragma once
+#include "common.h"
+
+enum { TP_EPI_NONE = 0, TP_EPI_SOFTCAP = 1, TP_EPI_GATED = 2 };
+
+struct GemmArgs {
+    const void* x; const void* w; void* y;
+    int in_dtype, out_dtype;
+    int M, N, K;            // N counts rows of W (for a gated product: 2 * padded units)
+    int epilogue; float cap;
+    int units;              // gated: columns of the output (the feed-forward width)
+    void* workspace; size_t workspace_bytes;
+    hipStream_t stream;
+};
+
+// plain tiled kernel, any dtype and shape; one fixed summation order per output element
+int gemm_simple_launch(const GemmArgs& a);
+// bf16 on the matrix cores: rows <= 64 (streams W once), and large row counts (LDS-tiled)
+bool gemm_skinny_supports(const GemmArgs& a);
+size_t gemm_skinny_workspace(const GemmArgs& a);
+int gemm_skinny_launch(const GemmArgs& a);
+bool gemm_mfma_supports(const GemmArgs& a);
+int gemm_mfma_launch(const GemmArgs& a);

@@ -1,0 +1,120 @@
+// Entry points of the matrix products and the plain tiled kernel.
+//
+// The plain kernel is the whole of the float32 path (no matrix-core mode, every output element summed
+// over k in index order whatever the batch is) and the fallback of the bf16 path for shapes the
+// matrix-core kernels refuse.  The reference's products are 4-bit codebook GEMVs
+// (runtime/cuda/codebook_gemv.cu:86-114); its only dense one is gemv_fp16_warp_k (cu:496-517).
+#include "gemm.h"
+
+template <typename TI, typename TO>
+__global__ void __launch_bounds__(256)
+gemm_simple_k(const TI* __restrict__ X, const TI* __restrict__ W, TO* __restrict__ Y, int M, int N, int K, float cap) {
+    __shared__ float xs[16][65];
+    __shared__ float ws[16][65];
+    const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
+    const int m0 = blockIdx.y * 64, n0 = blockIdx.x * 64;
+    float acc[4][4] = {};
+    for (int k0 = 0; k0 < K; k0 += 16) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int idx = tid + i * 256, r = idx >> 4, kk = idx & 15;
+            const int k = k0 + kk;
+            xs[kk][r] = (m0 + r < M && k < K) ? ld_f32(X + (size_t)(m0 + r) * K + k) : 0.f;
+            ws[kk][r] = (n0 + r < N && k < K) ? ld_f32(W + (size_t)(n0 + r) * K + k) : 0.f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < 16; kk++) {
+            float a[4], b[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) { a[i] = xs[kk][ty * 4 + i]; b[i] = ws[kk][tx * 4 + i]; }
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int m = m0 + ty * 4 + i;
+        if (m >= M) continue;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int n = n0 + tx * 4 + j;
+            if (n >= N) continue;
+            float v = acc[i][j];
+            if (cap > 0.f) v = softcap_f(v, cap);
+            st_f32(Y + (size_t)m * N + n, v);
+        }
+    }
+}
+
+extern "C" int tp_gated_act(const float* y, void* out, int dtype, int M, int I, void* stream);
+
+template <typename TI>
+static int simple_typed(const GemmArgs& a, void* y, int out_dtype, float cap) {
+    dim3 grid(tp_cdiv(a.N, 64), tp_cdiv(a.M, 64));
+    if (out_dtype == TP_F32)
+        gemm_simple_k<TI, float><<<grid, 256, 0, a.stream>>>((const TI*)a.x, (const TI*)a.w, (float*)y, a.M, a.N, a.K, cap);
+    else
+        gemm_simple_k<TI, bf16_t><<<grid, 256, 0, a.stream>>>((const TI*)a.x, (const TI*)a.w, (bf16_t*)y, a.M, a.N, a.K, cap);
+    return tp_check_launch("linear (plain kernel)");
+}
+
+int gemm_simple_launch(const GemmArgs& a) {
+    void* y = a.y;
+    int out_dtype = a.out_dtype;
+    if (a.epilogue == TP_EPI_GATED) {
+        TP_REQUIRE(a.workspace && a.workspace_bytes >= (size_t)a.M * a.N * 4, "gated product: workspace of %zu bytes is too small", a.workspace_bytes);
+        y = a.workspace;
+        out_dtype = TP_F32;
+    }
+    const float cap = a.epilogue == TP_EPI_SOFTCAP ? a.cap : 0.f;
+    int rc = a.in_dtype == TP_BF16 ? simple_typed<bf16_t>(a, y, out_dtype, cap) : simple_typed<float>(a, y, out_dtype, cap);
+    if (rc) return rc;
+    if (a.epilogue == TP_EPI_GATED) return tp_gated_act((const float*)y, a.y, a.out_dtype, a.M, a.units, a.stream);
+    return 0;
+}
+
+static int check_args(const GemmArgs& a) {
+    TP_REQUIRE(a.M > 0 && a.N > 0 && a.K > 0, "linear: empty shape M=%d N=%d K=%d", a.M, a.N, a.K);
+    TP_REQUIRE(a.in_dtype == TP_F32 || a.in_dtype == TP_BF16, "linear: unknown input dtype %d", a.in_dtype);
+    TP_REQUIRE(a.out_dtype == TP_F32 || a.out_dtype == TP_BF16, "linear: unknown output dtype %d", a.out_dtype);
+    TP_REQUIRE(!(a.in_dtype == TP_F32 && a.out_dtype == TP_BF16), "linear: float32 rows give float32 output");
+    TP_REQUIRE(a.epilogue != TP_EPI_SOFTCAP || a.cap > 0.f, "linear: a soft cap must be positive");
+    if (a.epilogue == TP_EPI_GATED) {
+        const int padded = 2 * ((a.units + 15) / 16) * 16;
+        TP_REQUIRE(a.units > 0 && a.N == padded, "gated product: %d units need a packed matrix of %d rows, found %d", a.units, padded, a.N);
+    }
+    return 0;
+}
+
+// algo: 0 = choose, 1 = plain, 2 = skinny matrix-core, 3 = tiled matrix-core
+static int pick(const GemmArgs& a, int algo) {
+    if (algo == 1) return 1;
+    if (algo == 2) return gemm_skinny_supports(a) ? 2 : -2;
+    if (algo == 3) return gemm_mfma_supports(a) ? 3 : -3;
+    if (gemm_skinny_supports(a)) return 2;
+    if (gemm_mfma_supports(a)) return 3;
+    return 1;
+}
+
+extern "C" long tp_linear_workspace_bytes(int in_dtype, int out_dtype, int M, int N, int K, int epilogue, int units, int algo) {
+    GemmArgs a{nullptr, nullptr, nullptr, in_dtype, out_dtype, M, N, K, epilogue, 1.f, units, nullptr, 0, nullptr};
+    const int p = pick(a, algo);
+    if (p == 2) return (long)gemm_skinny_workspace(a);
+    if (p == 1 && epilogue == TP_EPI_GATED) return (long)M * N * 4;
+    return 0;
+}
+
+extern "C" int tp_linear(const void* x, const void* w, void* y, int in_dtype, int out_dtype, int M, int N, int K,
+                         int epilogue, float cap, int units, void* workspace, long workspace_bytes, int algo, void* stream) {
+    GemmArgs a{x, w, y, in_dtype, out_dtype, M, N, K, epilogue, cap, units, workspace, (size_t)workspace_bytes, (hipStream_t)stream};
+    if (int rc = check_args(a)) return rc;
+    const int p = pick(a, algo);
+    TP_REQUIRE(p > 0, "linear: the requested kernel (%d) does not take M=%d N=%d K=%d dtype %d", algo, M, N, K, in_dtype);
+    if (p == 2) return gemm_skinny_launch(a);
+    if (p == 3) return gemm_mfma_launch(a);
+    return gemm_simple_launch(a);
+}

@@ -82,6 +82,11 @@ class StepContext:
     def page_table(self, group_index):
         return self._tables[group_index]
 
+    def max_keys(self, site):
+        """Most keys any sequence of this step can see at this cache site (a host number, for launch geometry)."""
+        longest = max(s + c for s, c in zip(self.starts, self.counts))
+        return min(longest, site.rows_cap) if site.rows_cap else longest
+
     # keys and values of this step, for entries that read another entry's cache during a prefill
     def mark_shared(self, entries):
         self._shared = set(entries)

@@ -70,10 +70,12 @@ class Attention(Mixer):
             else:
                 k, v = ctx.step_kv_of(ctx.cache_owner)
             out = ops.attention_prefill(q, k, v, H, KV, hd, ctx.cu_rows, ctx.max_count,
-                                        self.query_scale, self.softcap, self.window, ctx.dtype)
+                                        self.query_scale, self.softcap, self.window, ctx.dtype,
+                                        row_seq=ctx.row_seq, row_pos=ctx.row_pos)
         else:
             out = ops.attention_decode(q, H, KV, hd, ctx.new_len, table, site.k, site.v, rows_cap,
-                                       self.query_scale, self.softcap, self.window, ctx.dtype)
+                                       self.query_scale, self.softcap, self.window, ctx.dtype,
+                                       max_keys=ctx.max_keys(site))
         return ops.linear(out, self.w_o, ctx.dtype)
 
 
