@@ -32,6 +32,16 @@ class Runtime:
         self.ops = ops
         self._staging = []
         self._next = 0
+        self._widened = {}
+
+    def matrix(self, t):
+        """A stored floating-point tensor in the width the kernels compute in (bf16 widens to fp32 exactly)."""
+        if t.dtype == self.dtype:
+            return t
+        key = (t.data_ptr(), tuple(t.shape))
+        if key not in self._widened:          # a tied head and its embedding share one converted copy
+            self._widened[key] = (t, t.to(self.dtype))
+        return self._widened[key][1]
 
     def upload_i32(self, array):
         """Host int32 numpy array -> device tensor (asynchronous from pinned memory on a GPU)."""

@@ -108,10 +108,10 @@ class HipOps:
         """[2 * ceil16(I), K]: 16 rows of gate, the 16 rows of up of the same units, and so on; zero rows pad."""
         i, k = w_gate.shape
         ip = -(-i // GATE_GROUP) * GATE_GROUP
-        out = torch.zeros((ip // GATE_GROUP, 2, GATE_GROUP, k), dtype=w_gate.dtype, device=w_gate.device)
-        out[:, 0].reshape(ip, k)[:i] = w_gate
-        out[:, 1].reshape(ip, k)[:i] = w_up
-        return out.reshape(2 * ip, k)
+        out = torch.zeros((2, ip, k), dtype=w_gate.dtype, device=w_gate.device)
+        out[0, :i] = w_gate
+        out[1, :i] = w_up
+        return out.reshape(2, ip // GATE_GROUP, GATE_GROUP, k).transpose(0, 1).reshape(2 * ip, k).contiguous()
 
     # ---- row-wise kernels ----------------------------------------------------------------------------
     def embed_rows(self, tokens, table, scale):

@@ -45,9 +45,9 @@ class Attention(Mixer):
     def bind(self, tensors, rt):
         import torch
         self.rt = rt
-        self.w_qkv = torch.cat([tensors["q_proj.weight"], tensors["k_proj.weight"],
-                                tensors["v_proj.weight"]], dim=0).contiguous()
-        self.w_o = tensors["o_proj.weight"]
+        self.w_qkv = rt.matrix(torch.cat([tensors["q_proj.weight"], tensors["k_proj.weight"],
+                                          tensors["v_proj.weight"]], dim=0)).contiguous()
+        self.w_o = rt.matrix(tensors["o_proj.weight"])
         self.inv_freq = self.position.inv_freq(rt.device)
 
     def forward(self, ctx, x, site):

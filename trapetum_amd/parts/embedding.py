@@ -22,7 +22,7 @@ class ScaledEmbedding(Embedding):
 
     def bind(self, tensors, rt):
         self.rt = rt
-        self.table = tensors["weight"]
+        self.table = rt.matrix(tensors["weight"])
 
     def forward(self, ctx, tokens):
         return ctx.ops.embed_rows(tokens, self.table, self.scale)
@@ -39,7 +39,7 @@ class LinearHead(Head):
 
     def bind(self, tensors, rt):
         self.rt = rt
-        self.weight = tensors["weight"]
+        self.weight = rt.matrix(tensors["weight"])
 
     def forward(self, ctx, rows):
         import torch

@@ -24,8 +24,8 @@ class GatedMLP(FeedForward):
 
     def bind(self, tensors, rt):
         self.rt = rt
-        self.w_gate_up = rt.ops.pack_gate_up(tensors["gate_proj.weight"], tensors["up_proj.weight"])
-        self.w_down = tensors["down_proj.weight"]
+        self.w_gate_up = rt.ops.pack_gate_up(rt.matrix(tensors["gate_proj.weight"]), rt.matrix(tensors["up_proj.weight"]))
+        self.w_down = rt.matrix(tensors["down_proj.weight"])
 
     def forward(self, ctx, x):
         act = ctx.ops.gated_linear(x, self.w_gate_up, self.intermediate_size, self.activation, ctx.dtype)
