@@ -28,10 +28,64 @@ def classify(counts, starts):
         f"found counts {list(counts)} at lengths {list(starts)}")
 
 
+def step_arrays(cache, slots, counts, starts, want_rows, table_widths=None):
+    """The step's geometry as int32 arrays, in the order StepContext slices them."""
+    n, m = len(slots), int(sum(counts))
+    cu = np.zeros(n + 1, dtype=np.int64)
+    np.cumsum(counts, out=cu[1:])
+    row_seq = np.repeat(np.arange(n), counts)
+    row_pos = np.concatenate([np.arange(s, s + c) for s, c in zip(starts, counts)])
+    new_len = np.asarray(starts) + np.asarray(counts)
+    want = np.asarray(want_rows, dtype=np.int64)
+    if want.size and (want.min() < 0 or want.max() >= m):
+        raise StepError(f"wanted rows {list(want_rows)} reach outside the step's {m} rows")
+    parts = [np.asarray(slots), cu, row_seq, row_pos, new_len, want]
+    shapes = []
+    for gi in range(len(cache.kv_groups)):
+        t = cache.page_table(gi, slots, None if table_widths is None else table_widths[gi])
+        shapes.append(t.shape)
+        parts.append(t.reshape(-1))
+    flat = np.concatenate([np.asarray(p, dtype=np.int32).reshape(-1) for p in parts])
+    return flat, shapes
+
+
+class StaticStep:
+    """Fixed device memory for the geometry of decode steps of one batch size, so that a captured HIP graph
+    finds every step's numbers at the same addresses.  Page tables have the cache's widest width."""
+
+    RING = 8
+
+    def __init__(self, rt, cache, n_seq):
+        import torch
+        self.rt = rt
+        self.n_seq = n_seq
+        self.table_widths = [g.max_pages_per_seq for g in cache.kv_groups]
+        size = 6 * n_seq + 1 + sum(n_seq * w for w in self.table_widths)
+        self.size = size
+        self.device_buffer = torch.zeros(size, dtype=torch.int32, device=rt.device)
+        self.pinned = [torch.zeros(size, dtype=torch.int32, pin_memory=True) for _ in range(self.RING)]
+        self.events = [None] * self.RING
+        self.turn = 0
+
+    def fill(self, flat):
+        """Queue the copy of this step's numbers into the fixed buffer (on the current stream)."""
+        import torch
+        assert flat.size == self.size, (flat.size, self.size)
+        i = self.turn
+        self.turn = (i + 1) % self.RING
+        if self.events[i] is not None:
+            self.events[i].synchronize()
+        self.pinned[i].copy_(torch.from_numpy(flat))
+        self.device_buffer.copy_(self.pinned[i], non_blocking=True)
+        ev = torch.cuda.Event()
+        ev.record()
+        self.events[i] = ev
+
+
 class StepContext:
     """Everything parts need during a step.  Device tensors are int32."""
 
-    def __init__(self, rt, cache, slots, counts, starts, want_rows):
+    def __init__(self, rt, cache, slots, counts, starts, want_rows, static=None):
         self.rt = rt
         self.ops = rt.ops
         self.dtype = rt.dtype
@@ -45,24 +99,17 @@ class StepContext:
         self.max_count = max(self.counts)
         self.entry = None               # schedule entry now running
         self.cache_owner = None         # entry whose cache it uses
+        self.static = static
         self._shared = set()            # entries whose step keys/values a later entry reads
         self._step_kv = {}
         n, m = self.n_seq, self.n_rows
-        cu = np.zeros(n + 1, dtype=np.int64)
-        np.cumsum(self.counts, out=cu[1:])
-        row_seq = np.repeat(np.arange(n), self.counts)
-        row_pos = np.concatenate([np.arange(s, s + c) for s, c in zip(self.starts, self.counts)])
-        new_len = np.asarray(self.starts) + np.asarray(self.counts)
-        want = np.asarray(want_rows, dtype=np.int64)
-        if want.size and (want.min() < 0 or want.max() >= m):
-            raise StepError(f"wanted rows {want_rows} reach outside the step's {m} rows")
-        parts = [np.asarray(self.slots), cu, row_seq, row_pos, new_len, want]
-        tables = []
-        for gi, g in enumerate(cache.kv_groups):
-            tables.append(cache.page_table(gi, self.slots))
-            parts.append(tables[-1].reshape(-1))
-        flat = np.concatenate([np.asarray(p, dtype=np.int32).reshape(-1) for p in parts])
-        dev = rt.upload_i32(flat)
+        flat, shapes = step_arrays(cache, self.slots, self.counts, self.starts, want_rows,
+                                   static.table_widths if static is not None else None)
+        if static is not None:
+            static.fill(flat)
+            dev = static.device_buffer
+        else:
+            dev = rt.upload_i32(flat)
         o = 0
 
         def take(k):
@@ -75,15 +122,19 @@ class StepContext:
         self.row_seq = take(m)
         self.row_pos = take(m)
         self.new_len = take(n)
-        self.want_rows = take(want.size)
-        self.n_want = int(want.size)
-        self._tables = [take(t.size).reshape(t.shape) for t in tables]
+        self.n_want = len(want_rows)
+        self.identity_want = list(want_rows) == list(range(m))
+        self.want_rows = take(self.n_want)
+        self._tables = [take(int(np.prod(sh))).reshape(sh) for sh in shapes]
 
     def page_table(self, group_index):
         return self._tables[group_index]
 
     def max_keys(self, site):
-        """Most keys any sequence of this step can see at this cache site (a host number, for launch geometry)."""
+        """Most keys any sequence of this step can see at this cache site (a host number, for launch geometry).
+        With fixed step memory (a captured graph) it is the most the cache allows."""
+        if self.static is not None:
+            return site.rows_cap or self.cache.max_context
         longest = max(s + c for s, c in zip(self.starts, self.counts))
         return min(longest, site.rows_cap) if site.rows_cap else longest
 

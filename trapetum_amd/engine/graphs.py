@@ -1,0 +1,54 @@
+"""Decode steps replayed from captured HIP graphs, one graph per batch size.
+
+A decode step is some three hundred small launches; replaying them from a graph removes the host's share of
+the step (the reference reports the same lever for its own loop: runtime/README.md:49-58, and wraps capture
+and replay in `Graph`, runtime/src/lib.rs:1211-1236).  What changes from step to step (slots, positions,
+lengths, page tables, tokens) lives at fixed device addresses that are refilled before each replay; page
+tables have the cache's widest width, and launch geometry that depends on lengths is sized for the cache's
+context.  No memset node is recorded: buffers are filled by copies and kernels.
+"""
+import torch
+
+from .batch import StaticStep, StepContext, step_arrays
+
+
+class _Captured:
+    def __init__(self, static, tokens, ctx, graph, logits):
+        self.static, self.tokens, self.ctx, self.graph, self.logits = static, tokens, ctx, graph, logits
+
+
+class GraphedDecode:
+    def __init__(self, model, cache):
+        if model.rt.device.type != "cuda":
+            raise RuntimeError("HIP graphs need the GPU")
+        self.model = model
+        self.cache = cache
+        self.by_batch = {}
+
+    def step(self, slots, tokens):
+        """One decode step of the sequences in `slots` (a token each); returns fp32 logits [len(slots), vocab]
+        in memory that the next step of this batch size overwrites."""
+        model, cache = self.model, self.cache
+        counts, starts, want, tok = model.prepare(cache, slots, tokens)
+        if any(c != 1 for c in counts):
+            raise ValueError("graphed steps take one token per sequence")
+        b = len(slots)
+        cap = self.by_batch.get(b)
+        if cap is None:
+            static = StaticStep(model.rt, cache, b)
+            tokens_static = torch.zeros(b, dtype=torch.int32, device=model.rt.device)
+            tokens_static.copy_(tok)
+            ctx = StepContext(model.rt, cache, slots, counts, starts, want, static=static)
+            logits = model.run(ctx, tokens_static)          # this step, eagerly; also loads what capture must not
+            torch.cuda.synchronize(model.rt.device)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                captured_logits = model.run(ctx, tokens_static)
+            self.by_batch[b] = _Captured(static, tokens_static, ctx, graph, captured_logits)
+            return logits
+        flat, _ = step_arrays(cache, slots, counts, starts, want, cap.static.table_widths)
+        cap.static.fill(flat)
+        if tok.data_ptr() != cap.tokens.data_ptr():
+            cap.tokens.copy_(tok)
+        cap.graph.replay()
+        return cap.logits

@@ -6,12 +6,13 @@ operations as in the reference's forward (runtime/src/lib.rs:4553-4562): embed,
 each scheduled layer, final norm, head, final cap; the reference does this for one
 token of one sequence and always returns the whole logits vector.
 """
+import numpy as np
 import torch
 
 from ..cache.store import ModelCache
 from ..models.spec import ModelSpec
 from ..registry import build_part, part_class
-from .batch import StepContext, StepError
+from .batch import StepContext, StepError, classify
 
 
 class AssembledLayer:
@@ -100,6 +101,13 @@ class Model:
         want:   flat row indices whose logits are returned, in this order (default: each sequence's
                 last row).  Returns fp32 [len(want), vocab] on the device, or None when want is empty.
         """
+        counts, starts, want, tok = self.prepare(cache, slots, tokens, counts, want)
+        ctx = StepContext(self.rt, cache, slots, counts, starts, want)
+        return self.run(ctx, tok)
+
+    def prepare(self, cache, slots, tokens, counts=None, want=None):
+        """Check the step, reserve its cache rows, and bring the tokens to the device.  A refused step leaves
+        the cache as it was."""
         if not self.bound:
             raise RuntimeError("the model has no weights yet: load a folder or random weights first")
         n = len(slots)
@@ -107,11 +115,11 @@ class Model:
         if len(counts) != n:
             raise StepError(f"{n} slots but {len(counts)} counts")
         m = sum(counts)
+        host_tokens = None
         if isinstance(tokens, torch.Tensor):
             if tokens.dtype != torch.int32 or tokens.numel() != m:
                 raise StepError(f"token tensor must be int32 with {m} entries")
             tok = tokens.to(self.rt.device).reshape(-1)
-            host_tokens = None
         else:
             host_tokens = [int(t) for t in tokens]
             if len(host_tokens) != m:
@@ -124,21 +132,25 @@ class Model:
             for c in counts:
                 o += c
                 want.append(o - 1)
+        want = [int(w) for w in want]
+        if any(not 0 <= w < m for w in want):
+            raise StepError(f"wanted rows {want} reach outside the step's {m} rows")
         for s in slots:
             if s not in cache.book.length:
                 raise StepError(f"cache slot {s} is not in use")
         starts = [cache.length(s) for s in slots]
-        # decide the mode before the cache changes, so that a refused step leaves it untouched
-        from .batch import classify
-        classify(counts, starts)
+        classify(counts, starts)                 # before the cache changes
         cache.check_grow(slots, counts)
         for s, c in zip(slots, counts):
             cache.grow(s, c)
-        ctx = StepContext(self.rt, cache, slots, counts, starts, want)
-        ctx.mark_shared(self._shared)
         if host_tokens is not None:
-            import numpy as np
             tok = self.rt.upload_i32(np.asarray(host_tokens, dtype=np.int32))
+        return counts, starts, want, tok
+
+    def run(self, ctx, tok):
+        """The device work of a step (what a HIP graph captures): embed, layers, final norm, head."""
+        ctx.mark_shared(self._shared)
+        cache = ctx.cache
         stream = self.embedding.forward(ctx, tok)
         for i, e in enumerate(self.schedule):
             ctx.entry = i
@@ -146,6 +158,7 @@ class Model:
             stream = self.layers[e.layer].block.forward(ctx, stream, cache.site(ctx.cache_owner))
         if ctx.n_want == 0:
             return None
-        rows = stream if list(want) == list(range(m)) else ctx.ops.gather_rows(stream, ctx.want_rows)
+        whole = ctx.n_want == ctx.n_rows and ctx.identity_want
+        rows = stream if whole else ctx.ops.gather_rows(stream, ctx.want_rows)
         rows = self.final_norm.forward(ctx, rows)
         return self.head.forward(ctx, rows)

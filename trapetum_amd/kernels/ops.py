@@ -24,6 +24,8 @@ _CORE_SIGS = {
     "tp_attn_simple_prefill": [_P, _L, _P, _L, _P, _L, _I, _I, _I, _I, _I, _P, _P, _P, _F, _F, _I, _P, _P],
     "tp_attn_simple_decode": [_P, _L, _I, _I, _I, _I, _I, _P, _P, _I, _P, _P, _I, _I, _F, _F, _I, _P, _P],
     "tp_argmax": [_P, _I, _I, _P, _P],
+    "tp_repetition_penalty": [_P, _I, _I, _P, _I, _F, _P],
+    "tp_sample": [_P, _I, _I, _F, _I, _F, _P, _P, _P],
 }
 _ATTN_SIGS = {
     "tp_attn_prefill": [_P, _L, _P, _L, _P, _L, _I, _I, _I, _P, _I, _I, _F, _F, _I, _P, _P],
@@ -288,4 +290,25 @@ class HipOps:
             raise KernelError("argmax: logits must be contiguous float32 [rows, vocab]")
         out = torch.empty(logits.shape[0], dtype=torch.int32, device=self.device)
         self._call(self.lib, "tp_argmax", logits.data_ptr(), logits.shape[0], logits.shape[1], out.data_ptr(), self._stream())
+        return out
+
+    def apply_repetition_penalty(self, logits, recent, penalty):
+        """In place.  recent: int32 [rows, R], -1 where empty."""
+        self._dev(logits, recent)
+        if logits.dtype != torch.float32 or logits.dim() != 2 or not logits.is_contiguous():
+            raise KernelError("repetition_penalty: logits must be contiguous float32 [rows, vocab]")
+        if recent.dtype != torch.int32 or recent.dim() != 2 or recent.shape[0] != logits.shape[0] or not recent.is_contiguous():
+            raise KernelError("repetition_penalty: recent tokens must be contiguous int32 [rows, R]")
+        self._call(self.lib, "tp_repetition_penalty", logits.data_ptr(), logits.shape[0], logits.shape[1],
+                   recent.data_ptr(), recent.shape[1], float(penalty), self._stream())
+
+    def sample(self, logits, temperature, top_k, top_p, uniforms):
+        self._dev(logits, uniforms)
+        if logits.dtype != torch.float32 or logits.dim() != 2 or not logits.is_contiguous():
+            raise KernelError("sample: logits must be contiguous float32 [rows, vocab]")
+        if uniforms.dtype != torch.float32 or uniforms.numel() != logits.shape[0] or not uniforms.is_contiguous():
+            raise KernelError("sample: one float32 uniform number per row")
+        out = torch.empty(logits.shape[0], dtype=torch.int32, device=self.device)
+        self._call(self.lib, "tp_sample", logits.data_ptr(), logits.shape[0], logits.shape[1], float(temperature),
+                   int(top_k), float(top_p), uniforms.data_ptr(), out.data_ptr(), self._stream())
         return out

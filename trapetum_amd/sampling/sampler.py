@@ -1,0 +1,93 @@
+"""Choosing the next token: greedy, or the reference's temperature / top-p sampling.
+
+As the reference's next_tok (runtime/src/bin/serve.rs:41-72): temperature <= 0 is argmax with the smallest
+index winning ties (runtime/src/lib.rs:1376-1380); otherwise the top_k largest logits (256 there), softmax of
+(z - max) / T, the shortest prefix whose mass reaches top_p, and a draw r = u * kept mass walked down the
+sorted candidates.  A repetition penalty over the last 128 tokens, prompt included, comes first
+(serve.rs:285-294, :327-333).  The reference seeds one xorshift64 state from the clock (serve.rs:309-311);
+here every request owns a state derived from (seed, request index), so a request's draws do not depend on
+which other requests share its batch.  The logits never leave the device: only the chosen ids do.
+"""
+import collections
+import dataclasses
+
+import numpy as np
+import torch
+
+MASK64 = (1 << 64) - 1
+RECENT_WINDOW = 128          # tokens the repetition penalty looks back over (serve.rs:327)
+MAX_TOP_K = 1024
+
+
+@dataclasses.dataclass
+class SamplingParams:
+    temperature: float = 0.0            # 0 (or less): greedy
+    top_p: float = 0.95                 # the reference's default (serve.rs:1292)
+    top_k: int = 256                    # the reference keeps the 256 largest (serve.rs:52)
+    repetition_penalty: float = 1.0     # 1 (or less): off
+
+    def validate(self):
+        if not 1 <= self.top_k <= MAX_TOP_K:
+            raise ValueError(f"top_k {self.top_k} must lie in 1..{MAX_TOP_K}")
+        if not self.top_p > 0:
+            raise ValueError(f"top_p {self.top_p} must be positive")
+
+
+def xorshift64(state):
+    """One step of the reference's generator (serve.rs:63)."""
+    state ^= (state << 13) & MASK64
+    state ^= state >> 7
+    state ^= (state << 17) & MASK64
+    return state
+
+
+def initial_state(seed, index):
+    """A non-zero 64-bit state from (seed, request index): splitmix64 over their mix."""
+    z = (seed * 0x9E3779B97F4A7C15 + (index + 1) * 0xBF58476D1CE4E5B9) & MASK64
+    z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & MASK64
+    z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & MASK64
+    z ^= z >> 31
+    return z | 1
+
+
+class RequestSampling:
+    """What sampling remembers of one request."""
+
+    def __init__(self, seed, index, prompt):
+        self.state = initial_state(seed, index)
+        self.recent = collections.deque(prompt[-RECENT_WINDOW:], maxlen=RECENT_WINDOW)
+
+    def next_uniform(self):
+        self.state = xorshift64(self.state)
+        return float(np.float32((self.state >> 11) / float(1 << 53)))     # the reference draws in f32 (serve.rs:65)
+
+    def saw(self, token):
+        self.recent.append(token)
+
+
+class Sampler:
+    def __init__(self, rt, params):
+        params.validate()
+        self.rt = rt
+        self.params = params
+
+    def choose(self, logits, requests):
+        """logits fp32 [n, vocab] on the device (changed in place by a penalty); one RequestSampling per row.
+        Returns the chosen ids as a list, after which each request has seen its token."""
+        p = self.params
+        ops = self.rt.ops
+        if p.repetition_penalty > 1.0:
+            recent = np.full((len(requests), RECENT_WINDOW), -1, dtype=np.int32)
+            for i, r in enumerate(requests):
+                recent[i, :len(r.recent)] = list(r.recent)
+            ops.apply_repetition_penalty(logits, self.rt.upload_i32(recent), p.repetition_penalty)
+        if p.temperature <= 0:
+            ids = ops.argmax(logits)
+        else:
+            u = np.asarray([r.next_uniform() for r in requests], dtype=np.float32)
+            uniforms = self.rt.upload_i32(u.view(np.int32)).view(torch.float32)
+            ids = ops.sample(logits, p.temperature, p.top_k, p.top_p, uniforms)
+        out = [int(t) for t in ids.tolist()]
+        for r, t in zip(requests, out):
+            r.saw(t)
+        return out

@@ -25,7 +25,10 @@ def _seed_for(seed, name):
 class RandomWeights:
     """A weight source (names / shape / dtype / tensor) that draws each tensor when asked."""
 
-    def __init__(self, layout, seed, sigma=0.02, sigma_norm=0.1, store_dtype=torch.bfloat16):
+    def __init__(self, layout, seed, sigma=0.02, sigma_norm=0.1, store_dtype=torch.bfloat16, draw_on=None):
+        """draw_on: a device to draw on instead of the CPU (faster for large models; other values than the
+        CPU's for the same seed, so not what `write_model_folder` writes)."""
+        self.draw_on = draw_on
         self.layout = layout
         self.seed = seed
         self.sigma = sigma
@@ -51,6 +54,10 @@ class RandomWeights:
         if ts.init == "ones":
             return torch.ones(ts.shape, dtype=self.store_dtype)
         sigma = self.sigma_norm if ts.init == "norm" else self.sigma
+        if self.draw_on is not None:
+            gd = torch.Generator(device=self.draw_on).manual_seed(_seed_for(self.seed, name))
+            t = torch.empty(ts.shape, dtype=torch.float32, device=self.draw_on).normal_(0.0, 1.0, generator=gd)
+            return (t * sigma).to(self.store_dtype)
         t = torch.empty(ts.shape, dtype=torch.float32).normal_(0.0, 1.0, generator=g)
         return (t * sigma).to(self.store_dtype)
 
