@@ -1,0 +1,414 @@
+// bf16 attention on the matrix cores for one head size (compiled with -DTP_HD=<head_dim>, a multiple of 16 up
+// to 256): a prefill kernel over the step's own keys and values and a decode kernel over the paged cache.
+//
+// Formula as the reference's attn_k (runtime/cuda/codebook_gemv.cu:240-270): score = (q . k) * scale, then
+// cap * tanh(score / cap) if a cap is set, softmax over the visible keys in fp32, weighted sum of v, query head
+// h reading kv head h / (heads / kv_heads).  The scale is an argument (rsqrt(head_dim) in the reference), and a
+// window W hides keys with p - t >= W (the reference has none: runtime/src/lib.rs:4455).
+//
+// Both kernels compute scores transposed, S^T = K . Q^T with v_mfma_f32_16x16x32_bf16: key rows are the A
+// operand (a lane holds 8 consecutive elements of one key: one 16-byte load), queries the B operand, and a lane
+// ends up with 4 keys of ONE query, so the softmax statistics are per-lane scalars and the probabilities are
+// already laid out as the B operand of the second product.
+#include "common.h"
+#include "error_channel.h"
+
+#ifndef TP_HD
+#error "compile with -DTP_HD=<head_dim>"
+#endif
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
+
+namespace {
+constexpr int HD = TP_HD;
+constexpr int HDP = (HD + 31) / 32 * 32;       // head size padded to the product's k step
+constexpr int KSTEPS = HDP / 32;
+constexpr int NCH = HD / 8;                     // 16-byte chunks of a row
+static_assert(HD % 16 == 0 && HD >= 16 && HD <= 256, "head_dim must be a multiple of 16 up to 256");
+
+union Frag { uint4 u; bf16x8 v; bf16_t h[8]; };
+
+__device__ __forceinline__ bf16x8 ld_frag(const bf16_t* p, bool ok) {
+    Frag f;
+    if (ok) f.u = *reinterpret_cast<const uint4*>(p);
+    else f.u = make_uint4(0, 0, 0, 0);
+    return f.v;
+}
+__device__ __forceinline__ float score_of(float dot, float scale, float cap) {
+    float s = dot * scale;
+    if (cap > 0.f) s = cap * tanhf(s / cap);
+    return s;
+}
+}  // namespace
+
+// =====================================================================================================
+// prefill: every sequence of the step starts at position 0; keys and values are the step's own rows.
+// Block = 4 waves = 64 queries of one (sequence, head); each wave owns 16 queries.  Key tiles of 32 go
+// through LDS: K as stored (row = key), V transposed (row = head element) with the keys of a tile permuted
+// so that a lane's 8 probabilities meet the 8 values of the same keys in one 16-byte LDS read.
+// =====================================================================================================
+struct PrefillArgs {
+    const bf16_t* q; long q_stride; const bf16_t* k; long k_stride; const bf16_t* v; long v_stride;
+    int H, KV; const int* cu_rows; float scale, cap; int window; bf16_t* out;
+};
+
+namespace {
+constexpr int BKV = 32;
+constexpr int KLD = HDP + 8;                    // LDS row strides in elements: 16 bytes of padding spread the banks
+constexpr int VLD = BKV + 8;
+}
+
+__global__ void __launch_bounds__(256)
+attn_prefill_k(PrefillArgs a) {
+    __shared__ __attribute__((aligned(16))) bf16_t Ks[BKV * KLD];
+    __shared__ __attribute__((aligned(16))) bf16_t Vt[HD * VLD];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = lane & 15, g = lane >> 4;
+    const int seq = blockIdx.z, h = blockIdx.y, q0 = blockIdx.x * 64;
+    const int row0 = a.cu_rows[seq], T = a.cu_rows[seq + 1] - row0;
+    if (q0 >= T) return;
+    const int kvh = h / (a.H / a.KV);
+    const int qw0 = q0 + wave * 16, qpos = qw0 + c;
+    const bool q_ok = qpos < T;
+
+    bf16x8 qf[KSTEPS];
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ks++) {
+        const int d0 = ks * 32 + g * 8;
+        qf[ks] = ld_frag(a.q + (size_t)(row0 + (q_ok ? qpos : 0)) * a.q_stride + (size_t)h * HD + d0, q_ok && d0 < HD);
+    }
+    if (HDP > HD)                                   // the padding columns of K stay zero for the whole kernel
+        for (int i = tid; i < BKV * (HDP - HD); i += 256) Ks[(i / (HDP - HD)) * KLD + HD + i % (HDP - HD)] = 0;
+
+    f32x4 o[HD / 16];
+#pragma unroll
+    for (int dt = 0; dt < HD / 16; dt++) o[dt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    float m_i = -INFINITY, l_i = 0.f;
+
+    int k_lo = a.window > 0 ? max(0, q0 - a.window + 1) : 0;
+    k_lo &= ~(BKV - 1);
+    const int k_hi = min(T, q0 + 64);
+    for (int kt = k_lo; kt < k_hi; kt += BKV) {
+        __syncthreads();
+        for (int i = tid; i < BKV * NCH; i += 256) {
+            const int key = i / NCH, ch = i % NCH, tk = kt + key;
+            Frag kf, vf;
+            if (tk < T) {
+                kf.u = *reinterpret_cast<const uint4*>(a.k + (size_t)(row0 + tk) * a.k_stride + (size_t)kvh * HD + ch * 8);
+                vf.u = *reinterpret_cast<const uint4*>(a.v + (size_t)(row0 + tk) * a.v_stride + (size_t)kvh * HD + ch * 8);
+            } else {
+                kf.u = make_uint4(0, 0, 0, 0);
+                vf.u = make_uint4(0, 0, 0, 0);
+            }
+            *reinterpret_cast<uint4*>(Ks + key * KLD + ch * 8) = kf.u;
+            const int pos = ((key & 15) >> 2) * 8 + (key >> 4) * 4 + (key & 3);      // key = a*16 + g*4 + b -> g*8 + a*4 + b
+#pragma unroll
+            for (int e = 0; e < 8; e++) Vt[(ch * 8 + e) * VLD + pos] = vf.h[e];
+        }
+        __syncthreads();
+        const bool visible = qw0 < T && kt <= qw0 + 15 && !(a.window > 0 && kt + BKV - 1 < qw0 - a.window + 1);
+        if (!visible) continue;                      // wave-uniform: every key of the tile is hidden from the wave's queries
+
+        f32x4 s[2];
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            s[j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < KSTEPS; ks++) {
+                Frag kf;
+                kf.u = *reinterpret_cast<const uint4*>(Ks + (j * 16 + c) * KLD + ks * 32 + g * 8);
+                s[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qf[ks], s[j], 0, 0, 0);
+            }
+        }
+        // lane holds the scores of keys kt + j*16 + g*4 + i for its query qpos
+        float mx = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int tk = kt + j * 16 + g * 4 + i;
+                const bool ok = tk <= qpos && tk < T && (a.window <= 0 || qpos - tk < a.window);
+                const float v = ok ? score_of(s[j][i], a.scale, a.cap) : -INFINITY;
+                s[j][i] = v;
+                mx = fmaxf(mx, v);
+            }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(m_i, mx);
+        float alpha = 1.f, sum = 0.f;
+        Frag pf;
+        if (m_new == -INFINITY) {
+            pf.u = make_uint4(0, 0, 0, 0);
+        } else {
+            alpha = __expf(m_i - m_new);
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const float p = __expf(s[j][i] - m_new);
+                    sum += p;
+                    pf.h[j * 4 + i] = f32_to_bf16(p);
+                }
+        }
+        sum += __shfl_xor(sum, 16, 64);
+        sum += __shfl_xor(sum, 32, 64);
+        l_i = l_i * alpha + sum;
+        m_i = m_new;
+#pragma unroll
+        for (int dt = 0; dt < HD / 16; dt++) {
+            Frag vf;
+            vf.u = *reinterpret_cast<const uint4*>(Vt + (dt * 16 + c) * VLD + g * 8);
+            o[dt] = o[dt] * alpha;
+            o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf.v, o[dt], 0, 0, 0);
+        }
+    }
+    if (!q_ok) return;
+    const float inv = 1.f / l_i;
+    bf16_t* orow = a.out + ((size_t)(row0 + qpos) * a.H + h) * HD;
+#pragma unroll
+    for (int dt = 0; dt < HD / 16; dt++) {
+        ushort4 pk;
+        pk.x = f32_to_bf16(o[dt][0] * inv); pk.y = f32_to_bf16(o[dt][1] * inv);
+        pk.z = f32_to_bf16(o[dt][2] * inv); pk.w = f32_to_bf16(o[dt][3] * inv);
+        *reinterpret_cast<ushort4*>(orow + dt * 16 + g * 4) = pk;
+    }
+}
+
+extern "C" int tp_attn_prefill(const void* q, long q_stride, const void* k, long k_stride, const void* v, long v_stride,
+                               int M, int H, int KV, const int* cu_rows, int n_seq, int max_count,
+                               float scale, float cap, int window, void* out, void* stream) {
+    TP_REQUIRE(M > 0 && H > 0 && KV > 0 && n_seq > 0 && max_count > 0, "attention prefill: empty shape");
+    TP_REQUIRE(H % KV == 0, "attention: %d query heads are no multiple of %d kv heads", H, KV);
+    TP_REQUIRE(q_stride % 8 == 0 && k_stride % 8 == 0 && v_stride % 8 == 0 && (uintptr_t)q % 16 == 0 &&
+               (uintptr_t)k % 16 == 0 && (uintptr_t)v % 16 == 0, "attention prefill: rows must be 16-byte aligned");
+    TP_REQUIRE(H <= 65535 && n_seq <= 65535, "attention prefill: %d heads / %d sequences exceed one launch", H, n_seq);
+    PrefillArgs a{(const bf16_t*)q, q_stride, (const bf16_t*)k, k_stride, (const bf16_t*)v, v_stride, H, KV, cu_rows,
+                  scale, cap, window, (bf16_t*)out};
+    dim3 grid(tp_cdiv(max_count, 64), H, n_seq);
+    attn_prefill_k<<<grid, 256, 0, (hipStream_t)stream>>>(a);
+    return tp_check_launch("attention prefill");
+}
+
+// =====================================================================================================
+// decode: one query per sequence and head, keys and values in the paged cache.  A block owns one
+// (sequence, kv head, slice of the keys) and all the query heads of that kv head, so K and V are read once
+// for the group.  Scores by MFMA with key rows loaded straight from global memory; probabilities through
+// LDS; the weighted sum of V with plain FMAs (V's rows are contiguous along the head, not along the keys),
+// each thread owning one 16-byte chunk of the head for a subset of the keys.  Slices of the keys
+// (flash-decoding) write (max, sum, unnormalised output) to a workspace that a second kernel combines in
+// slice order.
+// =====================================================================================================
+struct DecodeArgs {
+    const bf16_t* q; long q_stride; int H, KV; const int* new_len; const int* table; int table_w;
+    const bf16_t* k_pool; const bf16_t* v_pool; int page, rows_cap; float scale, cap; int window;
+    bf16_t* out; float* ws_o; float* ws_ml; int nsplit;
+};
+
+namespace {
+constexpr int KB = 128;                          // keys per round of a block
+constexpr int KGROUPS = 256 / NCH;               // threads that share a chunk index walk the keys KGROUPS apart
+}
+
+template <int QT>
+__global__ void __launch_bounds__(256)
+attn_decode_k(DecodeArgs a) {
+    __shared__ float s_lds[QT][KB];
+    __shared__ float m_run[QT], l_run[QT], alpha_s[QT];
+    __shared__ float red[KGROUPS * HD];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = lane & 15, g = lane >> 4;
+    const int kvh = blockIdx.x, seq = blockIdx.y, split = blockIdx.z;
+    const int G = a.H / a.KV;
+    const int p = a.new_len[seq] - 1;
+    const int lo = a.window > 0 ? max(0, p - a.window + 1) : 0;
+    const int lo_al = lo & ~15;
+    int chunk = (p + 1 - lo_al + a.nsplit - 1) / a.nsplit;
+    chunk = (chunk + KB - 1) / KB * KB;
+    const int t_begin = lo_al + split * chunk;
+    const int t_end = min(p + 1, t_begin + chunk);
+    if (t_begin > p) {                               // this slice has no keys
+        if (tid < G) {
+            float* ml = a.ws_ml + (((size_t)seq * a.H + kvh * G + tid) * a.nsplit + split) * 2;
+            ml[0] = -INFINITY;
+            ml[1] = 0.f;
+        }
+        return;
+    }
+    const int* table = a.table + (size_t)seq * a.table_w;
+
+    bf16x8 qf[KSTEPS];
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ks++) {
+        const int d0 = ks * 32 + g * 8;
+        const bool ok = c < G && d0 < HD;
+        qf[ks] = ld_frag(a.q + (size_t)seq * a.q_stride + (size_t)(kvh * G + (ok ? c : 0)) * HD + (ok ? d0 : 0), ok);
+    }
+    if (tid < QT) { m_run[tid] = -INFINITY; l_run[tid] = 0.f; }
+    const int ch = tid % NCH, kg = tid / NCH;
+    const bool pv_thread = kg < KGROUPS;
+    float acc[QT][8];
+#pragma unroll
+    for (int qi = 0; qi < QT; qi++)
+#pragma unroll
+        for (int e = 0; e < 8; e++) acc[qi][e] = 0.f;
+    __syncthreads();
+
+    for (int t0 = t_begin; t0 < t_end; t0 += KB) {
+        // ---- scores of KB keys: wave w takes the 16-key tiles 2w and 2w + 1 -----------------------------
+#pragma unroll
+        for (int jj = 0; jj < 2; jj++) {
+            const int tile = wave * 2 + jj;
+            const int tb = t0 + tile * 16;
+            f32x4 s = (f32x4){0.f, 0.f, 0.f, 0.f};
+            if (tb < t_end) {                        // wave-uniform
+                int tk = tb + c;
+                tk = tk < lo ? lo : (tk > p ? p : tk);           // a row that exists; masked below
+                const int row = a.rows_cap > 0 ? tk % a.rows_cap : tk;
+                const int pg = table[row / a.page];
+                const bf16_t* kp = a.k_pool + (((size_t)pg * a.KV + kvh) * a.page + row % a.page) * HD;
+                bf16x8 kf[KSTEPS];
+#pragma unroll
+                for (int ks = 0; ks < KSTEPS; ks++) {
+                    const int d0 = ks * 32 + g * 8;
+                    kf[ks] = ld_frag(kp + (d0 < HD ? d0 : 0), d0 < HD);
+                }
+#pragma unroll
+                for (int ks = 0; ks < KSTEPS; ks++) s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[ks], qf[ks], s, 0, 0, 0);
+            }
+            if (c < QT) {
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int kl = tile * 16 + g * 4 + i, tk = t0 + kl;
+                    const bool ok = tk >= lo && tk < t_end;
+                    s_lds[c][kl] = ok ? score_of(s[i], a.scale, a.cap) : -INFINITY;
+                }
+            }
+        }
+        __syncthreads();
+        // ---- running softmax per query head: wave w takes heads w, w + 4, ... ---------------------------------
+        for (int qi = wave; qi < QT; qi += 4) {
+            const float v0 = s_lds[qi][lane], v1 = s_lds[qi][lane + 64];
+            const float mx = wave_max(fmaxf(v0, v1));
+            const float m_old = m_run[qi], m_new = fmaxf(m_old, mx);
+            float al = 1.f, p0 = 0.f, p1 = 0.f;
+            if (m_new != -INFINITY) {
+                al = __expf(m_old - m_new);
+                p0 = __expf(v0 - m_new);
+                p1 = __expf(v1 - m_new);
+            }
+            s_lds[qi][lane] = p0;
+            s_lds[qi][lane + 64] = p1;
+            const float sum = wave_sum(p0 + p1);
+            if (lane == 0) { m_run[qi] = m_new; l_run[qi] = l_run[qi] * al + sum; alpha_s[qi] = al; }
+        }
+        __syncthreads();
+        // ---- weighted sum of V: thread (chunk ch, key group kg) ------------------------------------------------
+        if (pv_thread) {
+#pragma unroll
+            for (int qi = 0; qi < QT; qi++) {
+                const float al = alpha_s[qi];
+#pragma unroll
+                for (int e = 0; e < 8; e++) acc[qi][e] *= al;
+            }
+            const int kmax = min(KB, t_end - t0);
+#pragma unroll 4
+            for (int kk = kg; kk < kmax; kk += KGROUPS) {
+                int tk = t0 + kk;
+                tk = tk < lo ? lo : tk;                          // hidden keys have probability 0
+                const int row = a.rows_cap > 0 ? tk % a.rows_cap : tk;
+                const int pg = table[row / a.page];
+                Frag vf;
+                vf.u = *reinterpret_cast<const uint4*>(a.v_pool + (((size_t)pg * a.KV + kvh) * a.page + row % a.page) * HD + ch * 8);
+                float vv[8];
+#pragma unroll
+                for (int e = 0; e < 8; e++) vv[e] = bf16_to_f32(vf.h[e]);
+#pragma unroll
+                for (int qi = 0; qi < QT; qi++) {
+                    const float pr = s_lds[qi][kk];
+#pragma unroll
+                    for (int e = 0; e < 8; e++) acc[qi][e] = fmaf(pr, vv[e], acc[qi][e]);
+                }
+            }
+        }
+        __syncthreads();
+    }
+    // ---- add the key groups' partial sums in group order and write ----------------------------------------------
+    for (int qi = 0; qi < QT; qi++) {
+        if (qi >= G) break;
+        if (pv_thread) {
+#pragma unroll
+            for (int e = 0; e < 8; e++) red[kg * HD + ch * 8 + e] = acc[qi][e];
+        }
+        __syncthreads();
+        if (tid < HD) {
+            float sum = 0.f;
+            for (int k2 = 0; k2 < KGROUPS; k2++) sum += red[k2 * HD + tid];
+            const int head = kvh * G + qi;
+            if (a.nsplit == 1) {
+                a.out[((size_t)seq * a.H + head) * HD + tid] = f32_to_bf16(sum / l_run[qi]);
+            } else {
+                const size_t at = ((size_t)seq * a.H + head) * a.nsplit + split;
+                a.ws_o[at * HD + tid] = sum;
+                if (tid == 0) { a.ws_ml[at * 2] = m_run[qi]; a.ws_ml[at * 2 + 1] = l_run[qi]; }
+            }
+        }
+        __syncthreads();
+    }
+}
+
+__global__ void attn_decode_combine_k(const float* __restrict__ ws_o, const float* __restrict__ ws_ml, int nsplit,
+                                      bf16_t* __restrict__ out) {
+    const size_t at = (size_t)blockIdx.x * nsplit;               // blockIdx.x = sequence * heads + head
+    float mx = -INFINITY;
+    for (int s = 0; s < nsplit; s++) mx = fmaxf(mx, ws_ml[(at + s) * 2]);
+    float den = 0.f;
+    for (int s = 0; s < nsplit; s++) {
+        const float m = ws_ml[(at + s) * 2];
+        if (m != -INFINITY) den += __expf(m - mx) * ws_ml[(at + s) * 2 + 1];
+    }
+    for (int d = threadIdx.x; d < HD; d += blockDim.x) {
+        float num = 0.f;
+        for (int s = 0; s < nsplit; s++) {
+            const float m = ws_ml[(at + s) * 2];
+            if (m != -INFINITY) num += __expf(m - mx) * ws_o[(at + s) * HD + d];
+        }
+        out[(size_t)blockIdx.x * HD + d] = f32_to_bf16(num / den);
+    }
+}
+
+extern "C" long tp_attn_decode_workspace_floats(int n_seq, int H, int nsplit) {
+    return nsplit > 1 ? (long)n_seq * H * nsplit * (HD + 2) : 0;
+}
+
+extern "C" int tp_attn_decode(const void* q, long q_stride, int n_seq, int H, int KV, const int* new_len,
+                              const int* table, int table_w, const void* k_pool, const void* v_pool, int page,
+                              int rows_cap, float scale, float cap, int window, void* out, void* workspace,
+                              int nsplit, void* stream) {
+    TP_REQUIRE(n_seq > 0 && H > 0 && KV > 0, "attention decode: empty shape");
+    TP_REQUIRE(H % KV == 0, "attention: %d query heads are no multiple of %d kv heads", H, KV);
+    const int G = H / KV;
+    TP_REQUIRE(G <= 16, "attention decode (matrix-core kernel): %d query heads per kv head exceed 16", G);
+    TP_REQUIRE(page > 0 && page % 16 == 0 && table_w > 0, "attention decode: page size %d must be a positive multiple of 16", page);
+    TP_REQUIRE(rows_cap >= 0 && rows_cap % page == 0, "attention decode: ring of %d rows is no multiple of the page size %d", rows_cap, page);
+    TP_REQUIRE(nsplit >= 1 && (nsplit == 1 || workspace), "attention decode: %d slices need a workspace", nsplit);
+    TP_REQUIRE(q_stride % 8 == 0 && (uintptr_t)q % 16 == 0, "attention decode: query rows must be 16-byte aligned");
+    TP_REQUIRE(KV <= 65535 * 1 && n_seq <= 65535 && nsplit <= 65535, "attention decode: grid too large");
+    DecodeArgs a{(const bf16_t*)q, q_stride, H, KV, new_len, table, table_w, (const bf16_t*)k_pool, (const bf16_t*)v_pool,
+                 page, rows_cap, scale, cap, window, (bf16_t*)out, nullptr, nullptr, nsplit};
+    if (nsplit > 1) {
+        a.ws_o = (float*)workspace;
+        a.ws_ml = a.ws_o + (size_t)n_seq * H * nsplit * HD;
+    }
+    dim3 grid(KV, n_seq, nsplit);
+    hipStream_t s = (hipStream_t)stream;
+    if (G <= 1) attn_decode_k<1><<<grid, 256, 0, s>>>(a);
+    else if (G <= 2) attn_decode_k<2><<<grid, 256, 0, s>>>(a);
+    else if (G <= 4) attn_decode_k<4><<<grid, 256, 0, s>>>(a);
+    else if (G <= 8) attn_decode_k<8><<<grid, 256, 0, s>>>(a);
+    else attn_decode_k<16><<<grid, 256, 0, s>>>(a);
+    if (int rc = tp_check_launch("attention decode")) return rc;
+    if (nsplit > 1) {
+        attn_decode_combine_k<<<n_seq * H, HD < 64 ? 64 : HD, 0, s>>>(a.ws_o, a.ws_ml, nsplit, (bf16_t*)out);
+        return tp_check_launch("attention decode (combine)");
+    }
+    return 0;
+}

@@ -1,22 +1,8 @@
 // Row-wise kernels: embedding, norms fused with the residual add, row gather, RoPE + cache write,
 // gated activation.  One block per row; statistics, angles and sums in fp32.
 #include "common.h"
-#include <string>
 
-// ---- error channel (defined once for the library) ----------------------------------------------
-static thread_local std::string g_error;
-extern "C" const char* tp_last_error() { return g_error.c_str(); }
-int tp_fail(const char* fmt, ...) {
-    char buf[1024];
-    va_list ap; va_start(ap, fmt); vsnprintf(buf, sizeof buf, fmt, ap); va_end(ap);
-    g_error = buf;
-    return 1;
-}
-int tp_check_launch(const char* what) {
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return tp_fail("%s: launch failed: %s", what, hipGetErrorString(e));
-    return 0;
-}
+#include "error_channel.h"
 
 // ---- embedding: out[r] = table[token[r]] * scale (fp32).  Reference: host gather of a pre-scaled fp16
 // row, runtime/src/lib.rs:4555, model/export_gemma.py:59-61. -----------------------------------------

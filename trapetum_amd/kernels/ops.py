@@ -278,6 +278,17 @@ class HipOps:
         if table.dtype != torch.int32 or table.dim() != 2 or table.shape[0] != n or not table.is_contiguous():
             raise KernelError("attention_decode: the page table must be contiguous int32 [sequences, pages]")
         out = torch.empty((n, H * hd), dtype=out_dtype, device=self.device)
+        if self._fast_attention(q.dtype, H, KV, hd) and k_pool.shape[2] % 16 == 0:
+            lib = self.attn_lib(hd)
+            keys = int(max_keys) if max_keys else k_pool.shape[0] * k_pool.shape[2]
+            nsplit = max(1, min(-(-512 // (n * KV)), -(-keys // 128), 64))
+            floats = lib.tp_attn_decode_workspace_floats(n, H, nsplit)
+            ws = torch.empty(floats, dtype=torch.float32, device=self.device) if floats else None
+            self._call(lib, "tp_attn_decode", q.data_ptr(), qs, n, H, KV, new_len.data_ptr(), table.data_ptr(),
+                       table.shape[1], k_pool.data_ptr(), v_pool.data_ptr(), k_pool.shape[2], rows_cap, float(scale),
+                       float(softcap), int(window), out.data_ptr(), ws.data_ptr() if ws is not None else None, nsplit,
+                       self._stream())
+            return out
         self._call(self.lib, "tp_attn_simple_decode", q.data_ptr(), qs, _code(q.dtype), n, H, KV, hd, new_len.data_ptr(),
                    table.data_ptr(), table.shape[1], k_pool.data_ptr(), v_pool.data_ptr(), k_pool.shape[2], rows_cap,
                    float(scale), float(softcap), int(window), out.data_ptr(), self._stream())
