@@ -1,0 +1,158 @@
+"""Toy parts defined by the tests, registered from outside the framework: a mixer with a state of fixed size
+per sequence, another position table, and an architecture that mixes them with the built-in parts.  They are
+no model of anyone's; they show that the framework's files need no change for a new part."""
+import dataclasses
+import math
+
+import torch
+
+from trapetum_amd.cache import StateSpec
+from trapetum_amd.config.base import ModelConfig, key
+from trapetum_amd.models.spec import LayerSpec, ModelSpec, ScheduleEntry, TensorSpec
+from trapetum_amd.parts import Mixer, Position
+from trapetum_amd.registry import register_architecture, register_part
+
+
+class EmaMixer(Mixer):
+    """state_t = decay * state_{t-1} + (1 - decay) * x_t per sequence; out_t = proj(state_t)."""
+
+    def __init__(self, hidden_size, decay):
+        self.hidden_size = hidden_size
+        self.decay = float(decay)
+
+    def tensor_specs(self):
+        return {"proj.weight": TensorSpec((self.hidden_size, self.hidden_size))}
+
+    def cache_spec(self):
+        return StateSpec((self.hidden_size,), "float32")
+
+    def bind(self, tensors, rt):
+        self.rt = rt
+        self.w = rt.matrix(tensors["proj.weight"])
+
+    def forward(self, ctx, x, site):
+        state = site.state                                   # [slots, hidden] fp32, zero for a fresh slot
+        out = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+        row = 0
+        for slot, count in zip(ctx.slots, ctx.counts):       # a scan over each sequence's rows of this step
+            s = state[slot]
+            for r in range(row, row + count):
+                s = self.decay * s + (1.0 - self.decay) * x[r].float()
+                out[r] = s
+            state[slot] = s
+            row += count
+        return ctx.ops.linear(out.to(ctx.dtype), self.w, ctx.dtype)
+
+
+class SquaredPosition(Position):
+    """Rotary frequencies d -> 1 / (1 + d)^2 over part of the head: another table through the same interface."""
+
+    def __init__(self, rotary_dim):
+        self.rotary_dim = rotary_dim
+
+    def inv_freq(self, device):
+        d = torch.arange(self.rotary_dim // 2, dtype=torch.float32)
+        return (1.0 / (1.0 + d) ** 2).to(device)
+
+
+@dataclasses.dataclass
+class ToyConfig(ModelConfig):
+    architecture = "ToyEmaForCausalLM"
+    n_layers: int = key("n_layers", "int")
+    width: int = key("width", "int")
+    heads: int = key("heads", "int")
+    head_size: int = key("head_size", "int")
+    ff_width: int = key("ff_width", "int")
+    vocab: int = key("vocab", "int")
+    eps: float = key("eps", "float")
+    decay: float = key("decay", "float")
+    rotary: int = key("rotary", "int")
+
+
+def toy_spec(c):
+    norm = ("rms_norm", {"size": c.width, "eps": c.eps, "weight_offset": 0.0})
+    layers = []
+    for l in range(c.n_layers):
+        p = f"blocks.{l}."
+        if l % 2 == 0:
+            mixer = ("toy_ema", {"hidden_size": c.width, "decay": c.decay})
+        else:
+            mixer = ("attention", {"hidden_size": c.width, "num_heads": c.heads, "num_kv_heads": c.heads,
+                                   "head_dim": c.head_size, "query_scale": 1.0 / math.sqrt(c.head_size),
+                                   "position": ("toy_squared", {"rotary_dim": c.rotary})})
+        ff = ("gated_mlp", {"hidden_size": c.width, "intermediate_size": c.ff_width, "activation": "gelu_tanh"})
+        layers.append(LayerSpec(block=("pre_norm", {}), mixer=mixer, feed_forward=ff, norm=norm,
+                                prefixes={"pre_mixer_norm": p + "n1.", "mixer": p + "mix.", "pre_ff_norm": p + "n2.",
+                                          "feed_forward": p + "ff."}))
+    # the order of running is data: layer 0 runs twice (its second run keeps a state of its own), and the
+    # last entry runs the attention layer again on the cache its first run filled
+    schedule = [ScheduleEntry(l) for l in range(c.n_layers)] + [ScheduleEntry(0), ScheduleEntry(1, cache_of=1)]
+    return ModelSpec(architecture=c.architecture, hidden_size=c.width, vocab_size=c.vocab,
+                     embedding=("scaled_embedding", {"vocab_size": c.vocab, "hidden_size": c.width, "scale": 1.0}),
+                     embedding_prefix="emb.", layers=layers, schedule=schedule, final_norm=norm, final_norm_prefix="out_norm.",
+                     head=("linear_head", {"vocab_size": c.vocab, "hidden_size": c.width, "softcap": None}),
+                     head_prefix="head.")
+
+
+def register():
+    register_part("mixer", "toy_ema", EmaMixer)
+    register_part("position", "toy_squared", SquaredPosition)
+    register_architecture(ToyConfig.architecture, ToyConfig, toy_spec)
+
+
+TOY = dict(n_layers=2, width=48, heads=3, head_size=16, ff_width=80, vocab=97, eps=1e-5, decay=0.8, rotary=8)
+
+
+# ---- the toy's own plain reference: whole sequences, float64, no cache ------------------------------------------------
+def toy_reference(cfg, W, tokens):
+    D = torch.float64
+    W = {k: v.to(D) for k, v in W.items()}
+    T = len(tokens)
+    x = W["emb.weight"][torch.tensor(tokens)]
+
+    def norm(t, w):
+        return t * torch.rsqrt((t * t).mean(-1, keepdim=True) + cfg["eps"]) * w
+
+    def gelu(g):
+        return 0.5 * g * (1 + torch.tanh(0.7978845608 * (g + 0.044715 * g ** 3)))
+
+    def ema(t, p):
+        s = torch.zeros(cfg["width"], dtype=D)
+        out = []
+        for r in range(T):
+            s = cfg["decay"] * s + (1 - cfg["decay"]) * t[r]
+            out.append(s)
+        return torch.stack(out) @ W[p + "mix.proj.weight"].T
+
+    def attn(t, p, kv=None):
+        H, hd, rot = cfg["heads"], cfg["head_size"], cfg["rotary"]
+        inv = 1.0 / (1.0 + torch.arange(rot // 2, dtype=D)) ** 2
+        ang = torch.arange(T, dtype=D)[:, None] * inv[None]
+        c, s = torch.cos(ang)[:, None], torch.sin(ang)[:, None]
+
+        def rope(u):
+            u = u.reshape(T, H, hd)
+            a, b = u[..., :rot // 2], u[..., rot // 2:rot]
+            return torch.cat([a * c - b * s, b * c + a * s, u[..., rot:]], -1)
+        q = rope(t @ W[p + "mix.q_proj.weight"].T)
+        if kv is None:
+            kv = (rope(t @ W[p + "mix.k_proj.weight"].T), (t @ W[p + "mix.v_proj.weight"].T).reshape(T, H, hd))
+        k, v = kv
+        sc = torch.einsum("thd,shd->hts", q, k) / math.sqrt(hd)
+        sc = sc.masked_fill(~torch.tril(torch.ones(T, T, dtype=torch.bool)), float("-inf"))
+        o = torch.einsum("hts,shd->thd", torch.softmax(sc, -1), v).reshape(T, H * hd)
+        return o @ W[p + "mix.o_proj.weight"].T, kv
+
+    kv1 = None
+    for l, reuse in [(0, False), (1, False), (0, False), (1, True)]:
+        p = f"blocks.{l}."
+        n = norm(x, W[p + "n1.weight"])
+        if l == 0:
+            x = x + ema(n, p)
+        else:
+            a, kv = attn(n, p, kv1 if reuse else None)
+            kv1 = kv1 or kv
+            x = x + a
+        n = norm(x, W[p + "n2.weight"])
+        x = x + (gelu(n @ W[p + "ff.gate_proj.weight"].T) * (n @ W[p + "ff.up_proj.weight"].T)) @ W[p + "ff.down_proj.weight"].T
+    return norm(x, W["out_norm.weight"]) @ W["head.weight"].T
