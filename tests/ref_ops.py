@@ -42,7 +42,7 @@ def add_rms_norm(stream, rows, gain_post, eps_post, gain_next, eps_next, out_dty
     return _norm(stream, gain_next, eps_next).to(out_dtype)
 
 
-def linear(x, w, out_dtype, softcap=None):
+def linear(x, w, out_dtype, softcap=None, defer=False):
     y = x.float() @ w.float().T
     if softcap:
         y = softcap * torch.tanh(y / softcap)
@@ -134,6 +134,10 @@ def attention_decode(q, H, KV, hd, new_len, table, k_pool, v_pool, rows_cap, sca
         for h in range(H):
             out[i, h * hd:(h + 1) * hd] = _attend(qf[i, h], keys[:, h // g], vals[:, h // g], scale, softcap)
     return out.to(out_dtype)
+
+
+def rows(r, dtype):
+    return r
 
 
 def gather_rows(x, rows):

@@ -64,6 +64,23 @@ def test_add_rms_norm(ops, dt, post, nxt, m, d):
         assert got is None
 
 
+@pytest.mark.parametrize("m,n,k", [(8, 2304, 2048), (3, 600, 9216), (64, 2304, 4096)])
+def test_deferred_product_into_add_rms_norm(ops, m, n, k):
+    """A product left in K slices and added by add_rms_norm equals the product, then the norm."""
+    from trapetum_amd.kernels.ops import SplitRows
+    x, w = randn(m, k, dtype=torch.bfloat16, seed=70), randn(n, k, dtype=torch.bfloat16, seed=71, scale=0.05)
+    rows = ops.linear(x, w, torch.bfloat16, defer=True)
+    assert isinstance(rows, SplitRows) and rows.shape == (m, n) and rows.slices.shape[0] > 1
+    ref_rows = x.cpu().double() @ w.cpu().double().T
+    assert rel_l2(ops.rows(rows, torch.float32), ref_rows) < 1e-5
+    stream = randn(m, n, seed=72)
+    gp, gn = 1.0 + randn(n, seed=73, scale=0.2), 1.0 + randn(n, seed=74, scale=0.2)
+    ref_stream = stream.cpu().clone()
+    ref = ref_ops.add_rms_norm(ref_stream, ref_rows.float(), gp.cpu(), 1e-6, gn.cpu(), 1e-6, torch.float32)
+    got = ops.add_rms_norm(stream, rows, gp, 1e-6, gn, 1e-6, torch.bfloat16)
+    assert rel_l2(stream, ref_stream) < 1e-5 and rel_l2(got, ref) < 6e-3
+
+
 def test_gather_rows(ops):
     x = randn(9, 88)
     rows = torch.tensor([8, 0, 3, 3], dtype=torch.int32, device=DEV)

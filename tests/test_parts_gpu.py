@@ -78,7 +78,7 @@ def test_gated_mlp(rt):
     w = bound(ff, rt, {"gate_proj.weight": rnd(200, 88, seed=3, scale=0.2), "up_proj.weight": rnd(200, 88, seed=4, scale=0.2),
                        "down_proj.weight": rnd(88, 200, seed=5, scale=0.2)})
     x = rnd(9, 88, seed=6).to(torch.bfloat16)
-    got = ff.forward(type("C", (), {"ops": rt.ops, "dtype": rt.dtype})(), act(rt, x))
+    got = rt.ops.rows(ff.forward(type("C", (), {"ops": rt.ops, "dtype": rt.dtype})(), act(rt, x)), rt.dtype)
     ref = plain.geglu(x.double(), w["gate_proj.weight"], w["up_proj.weight"], w["down_proj.weight"], lambda t: t)
     assert rel_l2(got, ref) < TOL[str(rt.dtype).split(".")[1]]
 
@@ -121,12 +121,12 @@ def test_attention_mixer_prefill_and_decode(rt):
     slots = [one.cache.acquire(), one.cache.acquire()]
     lens = [22, 5]
     ctx = one.step(slots, lens)
-    got = mixer.forward(ctx, act(rt, torch.cat([x[:n] for x, n in zip(seqs, lens)])), one.cache.site(0))
+    got = rt.ops.rows(mixer.forward(ctx, act(rt, torch.cat([x[:n] for x, n in zip(seqs, lens)])), one.cache.site(0)), rt.dtype)
     assert rel_l2(got[:22], refs[0][:22]) < tol and rel_l2(got[22:], refs[1][:5]) < tol
     for step in range(8):                                   # the second sequence ends after 4 more tokens
         live = [i for i in range(2) if lens[i] + step < seqs[i].shape[0]]
         ctx = one.step([slots[i] for i in live], [1] * len(live))
-        got = mixer.forward(ctx, act(rt, torch.stack([seqs[i][lens[i] + step] for i in live])), one.cache.site(0))
+        got = rt.ops.rows(mixer.forward(ctx, act(rt, torch.stack([seqs[i][lens[i] + step] for i in live])), one.cache.site(0)), rt.dtype)
         for j, i in enumerate(live):
             assert rel_l2(got[j], refs[i][lens[i] + step]) < 2 * tol, (step, i)
 
@@ -144,7 +144,7 @@ def test_window_edge_shows(rt):
     cfg = {"num_attention_heads": 6, "num_key_value_heads": 2, "head_dim": 32, "rope_theta": 1.0, "query_pre_attn_scalar": 1.0}
     one = OnePartContext(rt, mixer.cache_spec())
     s = one.cache.acquire()
-    got = mixer.forward(one.step([s], [20]), act(rt, x), one.cache.site(0))
+    got = rt.ops.rows(mixer.forward(one.step([s], [20]), act(rt, x), one.cache.site(0)), rt.dtype)
     q = (x.double() @ w["q_proj.weight"].T).reshape(20, 6, 32)
     k = (x.double() @ w["k_proj.weight"].T).reshape(20, 2, 32)
     v = (x.double() @ w["v_proj.weight"].T).reshape(20, 2, 32)
@@ -155,7 +155,7 @@ def test_window_edge_shows(rt):
     # the same edge, decoded token by token through the ring
     one2 = OnePartContext(rt, mixer.cache_spec())
     s = one2.cache.acquire()
-    rows = [mixer.forward(one2.step([s], [1]), act(rt, x[i:i + 1]), one2.cache.site(0)) for i in range(20)]
+    rows = [rt.ops.rows(mixer.forward(one2.step([s], [1]), act(rt, x[i:i + 1]), one2.cache.site(0)), rt.dtype) for i in range(20)]
     assert rel_l2(torch.cat(rows), ref) < tol
 
 
@@ -183,5 +183,12 @@ def test_sandwich_block(rt):
     one = OnePartContext(rt, block.mixer.cache_spec())
     s = one.cache.acquire()
     stream = x.to(DEV).clone()
-    out = block.forward(one.step([s], [13]), stream, one.cache.site(0))
-    assert out.dtype == torch.float32 and rel_l2(out, ref) < tol
+    out, nxt = block.forward(one.step([s], [13]), stream, one.cache.site(0))
+    assert nxt is None and out.dtype == torch.float32 and rel_l2(out, ref) < tol
+    # the next block's first norm, fused into this block's last add
+    follow = make_norm()
+    wf = bound(follow, rt, {"weight": rnd(88, seed=60, scale=0.3)})["weight"]
+    one = OnePartContext(rt, block.mixer.cache_spec())
+    s = one.cache.acquire()
+    out, nxt = block.forward(one.step([s], [13]), x.to(DEV).clone(), one.cache.site(0), next_norm=follow)
+    assert rel_l2(nxt, plain.rms_norm(ref, wf, 1e-5)) < max(tol, 3e-6)

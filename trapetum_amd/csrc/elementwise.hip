@@ -42,14 +42,48 @@ __global__ void rms_norm_k(const TI* __restrict__ x, const float* __restrict__ g
     for (int i = threadIdx.x; i < D; i += blockDim.x) st_f32(orow + i, (ld_f32(xr + i) * scale) * gain[i]);
 }
 
+// the same for rows of at most 256 * EPT elements: every element is read once and kept in registers
+template <typename TI, typename TO, int EPT>
+__global__ void __launch_bounds__(256)
+rms_norm_reg_k(const TI* __restrict__ x, const float* __restrict__ gain, float eps, TO* __restrict__ out, int D) {
+    __shared__ float red[16];
+    const TI* xr = x + (size_t)blockIdx.x * D;
+    TO* orow = out + (size_t)blockIdx.x * D;
+    float v[EPT], gn[EPT];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < EPT; j++) {
+        const int i = threadIdx.x + j * 256;
+        v[j] = i < D ? ld_f32(xr + i) : 0.f;
+        gn[j] = i < D ? gain[i] : 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < EPT; j++) ss += v[j] * v[j];
+    ss = block_sum(ss, red);
+    const float scale = rsqrtf(ss / (float)D + eps);
+#pragma unroll
+    for (int j = 0; j < EPT; j++) {
+        const int i = threadIdx.x + j * 256;
+        if (i < D) st_f32(orow + i, (v[j] * scale) * gn[j]);
+    }
+}
+
+template <typename TI, typename TO>
+static void rms_norm_launch(const void* x, const float* gain, float eps, void* out, int M, int D, hipStream_t s) {
+    if (D <= 256 * 4) rms_norm_reg_k<TI, TO, 4><<<M, 256, 0, s>>>((const TI*)x, gain, eps, (TO*)out, D);
+    else if (D <= 256 * 12) rms_norm_reg_k<TI, TO, 12><<<M, 256, 0, s>>>((const TI*)x, gain, eps, (TO*)out, D);
+    else if (D <= 256 * 20) rms_norm_reg_k<TI, TO, 20><<<M, 256, 0, s>>>((const TI*)x, gain, eps, (TO*)out, D);
+    else rms_norm_k<TI, TO><<<M, 256, 0, s>>>((const TI*)x, gain, eps, (TO*)out, D);
+}
+
 extern "C" int tp_rms_norm(const void* x, int in_dtype, const float* gain, float eps, void* out, int out_dtype,
                            int M, int D, void* stream) {
     TP_REQUIRE(M > 0 && D > 0, "rms_norm: empty shape M=%d D=%d", M, D);
     hipStream_t s = (hipStream_t)stream;
-    if (in_dtype == TP_F32 && out_dtype == TP_F32) rms_norm_k<float, float><<<M, 256, 0, s>>>((const float*)x, gain, eps, (float*)out, D);
-    else if (in_dtype == TP_F32 && out_dtype == TP_BF16) rms_norm_k<float, bf16_t><<<M, 256, 0, s>>>((const float*)x, gain, eps, (bf16_t*)out, D);
-    else if (in_dtype == TP_BF16 && out_dtype == TP_F32) rms_norm_k<bf16_t, float><<<M, 256, 0, s>>>((const bf16_t*)x, gain, eps, (float*)out, D);
-    else if (in_dtype == TP_BF16 && out_dtype == TP_BF16) rms_norm_k<bf16_t, bf16_t><<<M, 256, 0, s>>>((const bf16_t*)x, gain, eps, (bf16_t*)out, D);
+    if (in_dtype == TP_F32 && out_dtype == TP_F32) rms_norm_launch<float, float>(x, gain, eps, out, M, D, s);
+    else if (in_dtype == TP_F32 && out_dtype == TP_BF16) rms_norm_launch<float, bf16_t>(x, gain, eps, out, M, D, s);
+    else if (in_dtype == TP_BF16 && out_dtype == TP_F32) rms_norm_launch<bf16_t, float>(x, gain, eps, out, M, D, s);
+    else if (in_dtype == TP_BF16 && out_dtype == TP_BF16) rms_norm_launch<bf16_t, bf16_t>(x, gain, eps, out, M, D, s);
     else return tp_fail("rms_norm: unknown dtypes %d -> %d", in_dtype, out_dtype);
     return tp_check_launch("rms_norm");
 }
@@ -86,14 +120,79 @@ __global__ void add_rms_norm_k(float* __restrict__ stream, const T* __restrict__
     for (int i = threadIdx.x; i < D; i += blockDim.x) st_f32(orow + i, (sr[i] * scale_s) * gain_next[i]);   // own writes
 }
 
-extern "C" int tp_add_rms_norm(float* stream, const void* rows, int dtype, const float* gain_post, float eps_post,
-                               const float* gain_next, float eps_next, void* out, int M, int D, void* stream_) {
+// TR: type of the rows (float when they arrive as n_slices K slices of a product, each `slice_stride`
+// elements apart, added here in slice order); T: type of the normed output.
+template <typename TR, typename T, int EPT>
+__global__ void __launch_bounds__(256)
+add_rms_norm_reg_k(float* __restrict__ stream, const TR* __restrict__ rows, int n_slices, long slice_stride,
+                   const float* __restrict__ gain_post, float eps_post,
+                   const float* __restrict__ gain_next, float eps_next, T* __restrict__ out, int D) {
+    __shared__ float red[16];
+    float* sr = stream + (size_t)blockIdx.x * D;
+    const TR* ar = rows + (size_t)blockIdx.x * D;
+    float a[EPT], v[EPT], gp[EPT], gn[EPT];
+#pragma unroll
+    for (int j = 0; j < EPT; j++) {
+        const int i = threadIdx.x + j * 256;
+        const bool ok = i < D;
+        a[j] = ok ? ld_f32(ar + i) : 0.f;
+        for (int sl = 1; sl < n_slices; sl++) a[j] += ok ? ld_f32(ar + (size_t)sl * slice_stride + i) : 0.f;
+        v[j] = ok ? sr[i] : 0.f;
+        gp[j] = (ok && gain_post) ? gain_post[i] : 1.f;
+        gn[j] = (ok && gain_next) ? gain_next[i] : 0.f;
+    }
+    float scale_a = 1.f;
+    if (gain_post) {
+        float ss = 0.f;
+#pragma unroll
+        for (int j = 0; j < EPT; j++) ss += a[j] * a[j];
+        ss = block_sum(ss, red);
+        scale_a = rsqrtf(ss / (float)D + eps_post);
+    }
+    float ss2 = 0.f;
+#pragma unroll
+    for (int j = 0; j < EPT; j++) {
+        const int i = threadIdx.x + j * 256;
+        float t = a[j];
+        if (gain_post) t = (t * scale_a) * gp[j];
+        v[j] += t;
+        if (i < D) { sr[i] = v[j]; ss2 += v[j] * v[j]; }
+    }
+    if (!gain_next) return;
+    ss2 = block_sum(ss2, red);
+    const float scale_s = rsqrtf(ss2 / (float)D + eps_next);
+    T* orow = out + (size_t)blockIdx.x * D;
+#pragma unroll
+    for (int j = 0; j < EPT; j++) {
+        const int i = threadIdx.x + j * 256;
+        if (i < D) st_f32(orow + i, (v[j] * scale_s) * gn[j]);
+    }
+}
+
+template <typename TR, typename T>
+static int add_rms_norm_launch(float* stream, const void* rows, int n_slices, long slice_stride, const float* gp, float ep,
+                               const float* gn, float en, void* out, int M, int D, hipStream_t s) {
+    if (D <= 256 * 4) add_rms_norm_reg_k<TR, T, 4><<<M, 256, 0, s>>>(stream, (const TR*)rows, n_slices, slice_stride, gp, ep, gn, en, (T*)out, D);
+    else if (D <= 256 * 12) add_rms_norm_reg_k<TR, T, 12><<<M, 256, 0, s>>>(stream, (const TR*)rows, n_slices, slice_stride, gp, ep, gn, en, (T*)out, D);
+    else if (D <= 256 * 20) add_rms_norm_reg_k<TR, T, 20><<<M, 256, 0, s>>>(stream, (const TR*)rows, n_slices, slice_stride, gp, ep, gn, en, (T*)out, D);
+    else if (n_slices == 1 && sizeof(TR) == sizeof(T)) add_rms_norm_k<T><<<M, 256, 0, s>>>(stream, (const T*)rows, gp, ep, gn, en, (T*)out, D);
+    else return tp_fail("add_rms_norm: rows in slices need a width of at most %d, found %d", 256 * 20, D);
+    return 0;
+}
+
+extern "C" int tp_add_rms_norm(float* stream, const void* rows, int rows_dtype, int n_slices, long slice_stride,
+                               const float* gain_post, float eps_post, const float* gain_next, float eps_next,
+                               void* out, int out_dtype, int M, int D, void* stream_) {
     TP_REQUIRE(M > 0 && D > 0, "add_rms_norm: empty shape M=%d D=%d", M, D);
     TP_REQUIRE(!gain_next || out, "add_rms_norm: a next norm needs an output buffer");
+    TP_REQUIRE(n_slices >= 1 && (n_slices == 1 || rows_dtype == TP_F32), "add_rms_norm: rows in %d slices must be float32", n_slices);
     hipStream_t s = (hipStream_t)stream_;
-    if (dtype == TP_BF16) add_rms_norm_k<bf16_t><<<M, 256, 0, s>>>(stream, (const bf16_t*)rows, gain_post, eps_post, gain_next, eps_next, (bf16_t*)out, D);
-    else if (dtype == TP_F32) add_rms_norm_k<float><<<M, 256, 0, s>>>(stream, (const float*)rows, gain_post, eps_post, gain_next, eps_next, (float*)out, D);
-    else return tp_fail("add_rms_norm: unknown dtype %d", dtype);
+    int rc;
+    if (rows_dtype == TP_BF16 && out_dtype == TP_BF16) rc = add_rms_norm_launch<bf16_t, bf16_t>(stream, rows, n_slices, slice_stride, gain_post, eps_post, gain_next, eps_next, out, M, D, s);
+    else if (rows_dtype == TP_F32 && out_dtype == TP_F32) rc = add_rms_norm_launch<float, float>(stream, rows, n_slices, slice_stride, gain_post, eps_post, gain_next, eps_next, out, M, D, s);
+    else if (rows_dtype == TP_F32 && out_dtype == TP_BF16) rc = add_rms_norm_launch<float, bf16_t>(stream, rows, n_slices, slice_stride, gain_post, eps_post, gain_next, eps_next, out, M, D, s);
+    else return tp_fail("add_rms_norm: unsupported dtypes rows %d -> out %d", rows_dtype, out_dtype);
+    if (rc) return rc;
     return tp_check_launch("add_rms_norm");
 }
 

@@ -12,6 +12,7 @@ struct GemmArgs {
     int epilogue; float cap;
     int units;              // gated: columns of the output (the feed-forward width)
     void* workspace; size_t workspace_bytes;
+    int defer;              // split products: leave the K slices in the workspace [slices, M, N] for the consumer to add
     hipStream_t stream;
 };
 

@@ -101,7 +101,7 @@ static int pick(const GemmArgs& a, int algo) {
 }
 
 extern "C" long tp_linear_workspace_bytes(int in_dtype, int out_dtype, int M, int N, int K, int epilogue, int units, int algo) {
-    GemmArgs a{nullptr, nullptr, nullptr, in_dtype, out_dtype, M, N, K, epilogue, 1.f, units, nullptr, 0, nullptr};
+    GemmArgs a{nullptr, nullptr, nullptr, in_dtype, out_dtype, M, N, K, epilogue, 1.f, units, nullptr, 0, 0, nullptr};
     const int p = pick(a, algo);
     if (p == 2) return (long)gemm_skinny_workspace(a);
     if (p == 1 && epilogue == TP_EPI_GATED) return (long)M * N * 4;
@@ -109,8 +109,10 @@ extern "C" long tp_linear_workspace_bytes(int in_dtype, int out_dtype, int M, in
 }
 
 extern "C" int tp_linear(const void* x, const void* w, void* y, int in_dtype, int out_dtype, int M, int N, int K,
-                         int epilogue, float cap, int units, void* workspace, long workspace_bytes, int algo, void* stream) {
-    GemmArgs a{x, w, y, in_dtype, out_dtype, M, N, K, epilogue, cap, units, workspace, (size_t)workspace_bytes, (hipStream_t)stream};
+                         int epilogue, float cap, int units, void* workspace, long workspace_bytes, int defer,
+                         int algo, void* stream) {
+    GemmArgs a{x, w, y, in_dtype, out_dtype, M, N, K, epilogue, cap, units, workspace, (size_t)workspace_bytes, defer,
+               (hipStream_t)stream};
     if (int rc = check_args(a)) return rc;
     const int p = pick(a, algo);
     TP_REQUIRE(p > 0, "linear: the requested kernel (%d) does not take M=%d N=%d K=%d dtype %d", algo, M, N, K, in_dtype);

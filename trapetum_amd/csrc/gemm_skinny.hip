@@ -158,7 +158,7 @@ bool gemm_skinny_supports(const GemmArgs& a) {
 static void plan(const GemmArgs& a, int& nt, int& blocks, int& splits, int& k_per_split) {
     nt = a.epilogue == TP_EPI_GATED ? 2 : 1;
     blocks = tp_cdiv(a.N, 16 * nt);
-    int want = tp_cdiv(768, blocks);
+    int want = tp_cdiv(512, blocks);
     int most = a.K / 512;
     if (most < 1) most = 1;
     splits = want < most ? want : most;
@@ -199,7 +199,7 @@ int gemm_skinny_launch(const GemmArgs& a) {
     else if (a.M <= 32) launch_mt<2>(a, nt, grid, part, kps, splits);
     else launch_mt<4>(a, nt, grid, part, kps, splits);
     if (int rc = tp_check_launch("linear (skinny kernel)")) return rc;
-    if (splits > 1) {
+    if (splits > 1 && !a.defer) {
         const long total = (long)a.M * (a.epilogue == TP_EPI_GATED ? a.units : a.N);
         int rb = tp_cdiv(total, 256);
         if (rb > 2048) rb = 2048;

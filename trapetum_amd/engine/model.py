@@ -152,13 +152,26 @@ class Model:
         ctx.mark_shared(self._shared)
         cache = ctx.cache
         stream = self.embedding.forward(ctx, tok)
+        whole = ctx.n_want == ctx.n_rows and ctx.identity_want
+        normed = None
+        last = len(self.schedule) - 1
         for i, e in enumerate(self.schedule):
             ctx.entry = i
             ctx.cache_owner = i if e.cache_of is None else e.cache_of
-            stream = self.layers[e.layer].block.forward(ctx, stream, cache.site(ctx.cache_owner))
+            # the norm that meets the stream next, for this block to fuse into its last add
+            if i < last:
+                next_norm = self.layers[self.schedule[i + 1].layer].block.entry_norm()
+            else:
+                next_norm = self.final_norm if whole else None
+            if next_norm is not None and next_norm.gain is None:
+                next_norm = None
+            stream, normed = self.layers[e.layer].block.forward(ctx, stream, cache.site(ctx.cache_owner),
+                                                                 normed=normed, next_norm=next_norm)
         if ctx.n_want == 0:
             return None
-        whole = ctx.n_want == ctx.n_rows and ctx.identity_want
-        rows = stream if whole else ctx.ops.gather_rows(stream, ctx.want_rows)
-        rows = self.final_norm.forward(ctx, rows)
+        if whole and normed is not None:
+            rows = normed
+        else:
+            rows = stream if whole else ctx.ops.gather_rows(stream, ctx.want_rows)
+            rows = self.final_norm.forward(ctx, rows)
         return self.head.forward(ctx, rows)

@@ -16,11 +16,11 @@ _P, _I, _L, _F = _c.c_void_p, _c.c_int, _c.c_long, _c.c_float
 _CORE_SIGS = {
     "tp_embed_rows": [_P, _P, _I, _F, _P, _I, _I, _I, _P],
     "tp_rms_norm": [_P, _I, _P, _F, _P, _I, _I, _I, _P],
-    "tp_add_rms_norm": [_P, _P, _I, _P, _F, _P, _F, _P, _I, _I, _P],
+    "tp_add_rms_norm": [_P, _P, _I, _I, _L, _P, _F, _P, _F, _P, _I, _I, _I, _P],
     "tp_gather_rows": [_P, _P, _P, _I, _I, _I, _P],
     "tp_rope_kv_write": [_P, _L, _P, _L, _P, _L, _I, _I, _I, _I, _I, _P, _I, _P, _P, _P, _P, _I, _P, _P, _I, _I, _P],
     "tp_gated_act": [_P, _P, _I, _I, _I, _P],
-    "tp_linear": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P, _L, _I, _P],
+    "tp_linear": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P, _L, _I, _I, _P],
     "tp_attn_simple_prefill": [_P, _L, _P, _L, _P, _L, _I, _I, _I, _I, _I, _P, _P, _P, _F, _F, _I, _P, _P],
     "tp_attn_simple_decode": [_P, _L, _I, _I, _I, _I, _I, _P, _P, _I, _P, _P, _I, _I, _F, _F, _I, _P, _P],
     "tp_argmax": [_P, _I, _I, _P, _P],
@@ -39,6 +39,16 @@ GATE_GROUP = 16
 
 class KernelError(RuntimeError):
     """A kernel refused its operands, or the library could not be loaded."""
+
+
+class SplitRows:
+    """Rows of a product still in K slices: fp32 [slices, M, N], to be added in slice order by the kernel that
+    consumes them (`add_rms_norm`), which saves a launch and a rounding.  `HipOps.rows()` adds them otherwise."""
+
+    def __init__(self, slices):
+        self.slices = slices
+        self.shape = tuple(slices.shape[1:])
+        self.dtype = torch.float32
 
 
 def _code(dtype):
@@ -141,8 +151,13 @@ class HipOps:
         return out
 
     def add_rms_norm(self, stream, rows, gain_post, eps_post, gain_next, eps_next, out_dtype):
-        self._dev(stream, rows, gain_post, gain_next)
+        """stream += post-norm(rows) (or rows); returns next-norm(stream) or None.  rows: a tensor or SplitRows."""
         m, d = stream.shape
+        n_slices, stride = 1, 0
+        if isinstance(rows, SplitRows):
+            n_slices, stride = rows.slices.shape[0], rows.slices.stride(0)
+            rows = rows.slices[0]
+        self._dev(stream, rows, gain_post, gain_next)
         if stream.dtype != torch.float32 or not stream.is_contiguous():
             raise KernelError("add_rms_norm: the stream must be contiguous float32")
         if tuple(rows.shape) != (m, d) or not rows.is_contiguous():
@@ -150,16 +165,18 @@ class HipOps:
         for g in (gain_post, gain_next):
             if g is not None and (g.dtype != torch.float32 or g.numel() != d or not g.is_contiguous()):
                 raise KernelError(f"add_rms_norm: gains must be float32 [{d}]")
-        out = None
-        if gain_next is not None:
-            if out_dtype != rows.dtype:
-                raise KernelError("add_rms_norm: the next norm's output has the dtype of the rows")
-            out = torch.empty((m, d), dtype=out_dtype, device=self.device)
-        self._call(self.lib, "tp_add_rms_norm", stream.data_ptr(), rows.data_ptr(), _code(rows.dtype),
+        out = torch.empty((m, d), dtype=out_dtype, device=self.device) if gain_next is not None else None
+        self._call(self.lib, "tp_add_rms_norm", stream.data_ptr(), rows.data_ptr(), _code(rows.dtype), n_slices, stride,
                    gain_post.data_ptr() if gain_post is not None else None, float(eps_post),
                    gain_next.data_ptr() if gain_next is not None else None, float(eps_next),
-                   out.data_ptr() if out is not None else None, m, d, self._stream())
+                   out.data_ptr() if out is not None else None, _code(out_dtype), m, d, self._stream())
         return out
+
+    def rows(self, rows, dtype):
+        """A tensor of `dtype` from what `linear` returned."""
+        if isinstance(rows, SplitRows):
+            return rows.slices.sum(dim=0).to(dtype)
+        return rows
 
     def gather_rows(self, x, rows):
         self._dev(x, rows)
@@ -205,7 +222,7 @@ class HipOps:
                    page, rows_cap, self._stream())
 
     # ---- matrix products -----------------------------------------------------------------------------
-    def _linear(self, x, w, out_dtype, epilogue, cap, units):
+    def _linear(self, x, w, out_dtype, epilogue, cap, units, defer=False):
         self._dev(x, w)
         if x.dim() != 2 or w.dim() != 2 or not x.is_contiguous() or not w.is_contiguous():
             raise KernelError("linear: rows and matrix must be contiguous 2-D tensors")
@@ -216,19 +233,26 @@ class HipOps:
         if w.shape[1] != k:
             raise KernelError(f"linear: rows have {k} columns, the matrix {w.shape[1]}")
         cols = units if epilogue == EPI_GATED else n
-        out = torch.empty((m, cols), dtype=out_dtype, device=self.device)
         algo = self.force_linear
         nbytes = self.lib.tp_linear_workspace_bytes(_code(x.dtype), _code(out_dtype), m, n, k, epilogue, units, algo)
+        if defer and epilogue == EPI_NONE and nbytes and nbytes % (m * n * 4) == 0 and nbytes // (m * n * 4) > 1:
+            slices = torch.empty((nbytes // (m * n * 4), m, n), dtype=torch.float32, device=self.device)
+            self._call(self.lib, "tp_linear", x.data_ptr(), w.data_ptr(), None, _code(x.dtype), _code(out_dtype),
+                       m, n, k, epilogue, float(cap), units, slices.data_ptr(), nbytes, 1, algo, self._stream())
+            return SplitRows(slices)
+        out = torch.empty((m, cols), dtype=out_dtype, device=self.device)
         ws = torch.empty(nbytes, dtype=torch.uint8, device=self.device) if nbytes else None
         self._call(self.lib, "tp_linear", x.data_ptr(), w.data_ptr(), out.data_ptr(), _code(x.dtype), _code(out_dtype),
-                   m, n, k, epilogue, float(cap), units, ws.data_ptr() if ws is not None else None, nbytes, algo,
+                   m, n, k, epilogue, float(cap), units, ws.data_ptr() if ws is not None else None, nbytes, 0, algo,
                    self._stream())
         return out
 
-    def linear(self, x, w, out_dtype, softcap=None):
+    def linear(self, x, w, out_dtype, softcap=None, defer=False):
+        """x @ w^T.  defer: the caller hands the result to `add_rms_norm` (or through `rows()`), so a product
+        computed in K slices may come back as SplitRows."""
         if softcap:
             return self._linear(x, w, out_dtype, EPI_SOFTCAP, softcap, 0)
-        return self._linear(x, w, out_dtype, EPI_NONE, 0.0, 0)
+        return self._linear(x, w, out_dtype, EPI_NONE, 0.0, 0, defer=defer)
 
     def gated_linear(self, x, w_packed, inter, activation, out_dtype):
         if activation != "gelu_tanh":

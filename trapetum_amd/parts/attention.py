@@ -76,7 +76,7 @@ class Attention(Mixer):
             out = ops.attention_decode(q, H, KV, hd, ctx.new_len, table, site.k, site.v, rows_cap,
                                        self.query_scale, self.softcap, self.window, ctx.dtype,
                                        max_keys=ctx.max_keys(site))
-        return ops.linear(out, self.w_o, ctx.dtype)
+        return ops.linear(out, self.w_o, ctx.dtype, defer=True)
 
 
 register_part("mixer", "attention", Attention)

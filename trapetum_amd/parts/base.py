@@ -11,8 +11,13 @@ step (`forward`).  Interfaces:
   Mixer        cache_spec() -> KVSpec | StateSpec | None;
                forward(ctx, x, site) -> rows [M, hidden], x being the normed rows.
   FeedForward  forward(ctx, x) -> rows [M, hidden].
-  Block        sites() -> names of its norms;  forward(ctx, stream) -> stream, the
-               residual stream being fp32 [M, hidden].
+               (A mixer or feed-forward may return what `ops.linear(..., defer=True)` gave it: the block
+               hands it to `ops.add_rms_norm`, or turns it into a tensor with `ops.rows`.)
+  Block        norm_sites() -> names of its norms;  forward(ctx, stream, site, normed, next_norm)
+               -> (stream, normed_next), the residual stream being fp32 [M, hidden].  entry_norm()
+               names the norm the block applies to the stream first (or None); the block that ran
+               before may already have applied it (`normed`), fused into its last add, and this block
+               may do the same for the next one (`next_norm` -> `normed_next`, else None).
   Embedding    forward(ctx, tokens) -> fp32 stream;  Head  forward(ctx, rows) -> fp32 logits.
 
 `ctx` is the step's StepContext: batch geometry on the device, the kernels
@@ -67,7 +72,10 @@ class Block(Part):
     def norm_sites(cls):
         return ()
 
-    def forward(self, ctx, stream, site):
+    def entry_norm(self):
+        return None
+
+    def forward(self, ctx, stream, site, normed=None, next_norm=None):
         raise NotImplementedError
 
 

@@ -7,7 +7,9 @@ pre_norm  x += mixer(pre_mixer_norm(x));  x += ff(pre_ff_norm(x))
 
 The stream is fp32 and the sum is formed in fp32 (the reference adds in fp32 and
 stores fp16: runtime/cuda/codebook_gemv.cu:539-542).  Where a norm of a sub-layer's
-output is followed by the add and by the next norm, one kernel does all three.
+output is followed by the add and by the next norm, one kernel does all three; that
+includes the first norm of the block that runs next (`next_norm`), whose result the
+next block receives as `normed`.
 """
 from ..registry import register_part
 from .base import Block
@@ -21,6 +23,7 @@ def add_then_norm(ctx, stream, rows, post, nxt):
         return ctx.ops.add_rms_norm(stream, rows,
                                     post.gain if post else None, post.eps if post else 0.0,
                                     nxt.gain if nxt else None, nxt.eps if nxt else 0.0, ctx.dtype)
+    rows = ctx.ops.rows(rows, ctx.dtype)
     if post is not None:
         rows = post.forward(ctx, rows)
     ctx.ops.add_rms_norm(stream, rows, None, 0.0, None, 0.0, ctx.dtype)
@@ -32,14 +35,16 @@ class SandwichBlock(Block):
     def norm_sites(cls):
         return ("pre_mixer_norm", "post_mixer_norm", "pre_ff_norm", "post_ff_norm")
 
-    def forward(self, ctx, stream, site):
+    def entry_norm(self):
+        return self.norms["pre_mixer_norm"]
+
+    def forward(self, ctx, stream, site, normed=None, next_norm=None):
         n = self.norms
-        x = n["pre_mixer_norm"].forward(ctx, stream)
+        x = normed if normed is not None else n["pre_mixer_norm"].forward(ctx, stream)
         a = self.mixer.forward(ctx, x, site)
         x = add_then_norm(ctx, stream, a, n["post_mixer_norm"], n["pre_ff_norm"])
         m = self.feed_forward.forward(ctx, x)
-        add_then_norm(ctx, stream, m, n["post_ff_norm"], None)
-        return stream
+        return stream, add_then_norm(ctx, stream, m, n["post_ff_norm"], next_norm)
 
 
 class PreNormBlock(Block):
@@ -47,14 +52,16 @@ class PreNormBlock(Block):
     def norm_sites(cls):
         return ("pre_mixer_norm", "pre_ff_norm")
 
-    def forward(self, ctx, stream, site):
+    def entry_norm(self):
+        return self.norms["pre_mixer_norm"]
+
+    def forward(self, ctx, stream, site, normed=None, next_norm=None):
         n = self.norms
-        x = n["pre_mixer_norm"].forward(ctx, stream)
+        x = normed if normed is not None else n["pre_mixer_norm"].forward(ctx, stream)
         a = self.mixer.forward(ctx, x, site)
         x = add_then_norm(ctx, stream, a, None, n["pre_ff_norm"])
         m = self.feed_forward.forward(ctx, x)
-        add_then_norm(ctx, stream, m, None, None)
-        return stream
+        return stream, add_then_norm(ctx, stream, m, None, next_norm)
 
 
 register_part("block", "sandwich", SandwichBlock)

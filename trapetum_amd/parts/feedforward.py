@@ -29,7 +29,7 @@ class GatedMLP(FeedForward):
 
     def forward(self, ctx, x):
         act = ctx.ops.gated_linear(x, self.w_gate_up, self.intermediate_size, self.activation, ctx.dtype)
-        return ctx.ops.linear(act, self.w_down, ctx.dtype)
+        return ctx.ops.linear(act, self.w_down, ctx.dtype, defer=True)
 
 
 register_part("feed_forward", "gated_mlp", GatedMLP)
