@@ -193,8 +193,10 @@ extern "C" int tp_attn_prefill(const void* q, long q_stride, const void* k, long
 // decode: one query per sequence and head, keys and values in the paged cache.  A block owns one
 // (sequence, kv head, slice of the keys) and all the query heads of that kv head, so K and V are read once
 // for the group.  Scores by MFMA with key rows loaded straight from global memory; probabilities through
-// LDS; the weighted sum of V with plain FMAs (V's rows are contiguous along the head, not along the keys),
-// each thread owning one 16-byte chunk of the head for a subset of the keys.  Slices of the keys
+// a wave's LDS; the weighted sum of V with plain FMAs (V's rows are contiguous along the head, not along the
+// keys), each lane owning one 16-byte chunk of the head for a subset of the wave's 16 keys.  A wave keeps its
+// own running softmax over the keys it sees, so the waves of a block meet only once, at the end; a round's value
+// chunks are fetched together with its key rows, before the scores are known, so the two latencies overlap.  Slices of the keys
 // (flash-decoding) write (max, sum, unnormalised output) to a workspace that a second kernel combines in
 // slice order.
 // =====================================================================================================
@@ -205,16 +207,19 @@ struct DecodeArgs {
 };
 
 namespace {
-constexpr int KB = 128;                          // keys per round of a block
-constexpr int KGROUPS = 256 / NCH;               // threads that share a chunk index walk the keys KGROUPS apart
+constexpr int DTH = 256;                         // 4 waves; each scores and sums its own 16 keys of a round
+constexpr int ROUND = 64;                        // keys a block takes per round
+constexpr int KGW = 64 / NCH > 16 ? 16 : 64 / NCH;   // key groups of a wave: lanes with one chunk index walk the keys KGW apart
+constexpr int VPT = (16 + KGW - 1) / KGW;        // value chunks a lane fetches per round
 }
 
 template <int QT>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(DTH)
 attn_decode_k(DecodeArgs a) {
-    __shared__ float s_lds[QT][KB];
-    __shared__ float m_run[QT], l_run[QT], alpha_s[QT];
-    __shared__ float red[KGROUPS * HD];
+    __shared__ float p_lds[4][QT][16];               // a wave's probabilities of its 16 keys
+    __shared__ float alpha_lds[4][QT];
+    __shared__ float m_w[4][QT], l_w[4][QT];
+    __shared__ float red[4 * KGW * HD];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = lane & 15, g = lane >> 4;
     const int kvh = blockIdx.x, seq = blockIdx.y, split = blockIdx.z;
     const int G = a.H / a.KV;
@@ -222,10 +227,10 @@ attn_decode_k(DecodeArgs a) {
     const int lo = a.window > 0 ? max(0, p - a.window + 1) : 0;
     const int lo_al = lo & ~15;
     int chunk = (p + 1 - lo_al + a.nsplit - 1) / a.nsplit;
-    chunk = (chunk + KB - 1) / KB * KB;
+    chunk = (chunk + ROUND - 1) / ROUND * ROUND;
     const int t_begin = lo_al + split * chunk;
     const int t_end = min(p + 1, t_begin + chunk);
-    if (t_begin > p) {                               // this slice has no keys
+    if (t_begin > p) {                               // this slice has no keys (only when there are several)
         if (tid < G) {
             float* ml = a.ws_ml + (((size_t)seq * a.H + kvh * G + tid) * a.nsplit + split) * 2;
             ml[0] = -INFINITY;
@@ -242,113 +247,127 @@ attn_decode_k(DecodeArgs a) {
         const bool ok = c < G && d0 < HD;
         qf[ks] = ld_frag(a.q + (size_t)seq * a.q_stride + (size_t)(kvh * G + (ok ? c : 0)) * HD + (ok ? d0 : 0), ok);
     }
-    if (tid < QT) { m_run[tid] = -INFINITY; l_run[tid] = 0.f; }
-    const int ch = tid % NCH, kg = tid / NCH;
-    const bool pv_thread = kg < KGROUPS;
+    // the lane's part in the weighted sum: chunk ch of the head, keys kgw, kgw + KGW, ... of the wave's 16
+    const int ch = lane % NCH, kgw = lane / NCH;
+    const bool pv_lane = kgw < KGW;
     float acc[QT][8];
 #pragma unroll
     for (int qi = 0; qi < QT; qi++)
 #pragma unroll
         for (int e = 0; e < 8; e++) acc[qi][e] = 0.f;
-    __syncthreads();
+    float m_run = -INFINITY, l_run = 0.f;            // of query head c, over this wave's keys so far
 
-    for (int t0 = t_begin; t0 < t_end; t0 += KB) {
-        // ---- scores of KB keys: wave w takes the 16-key tiles 2w and 2w + 1 -----------------------------
+    for (int tb = t_begin + wave * 16; tb < t_end; tb += ROUND) {
+        // ---- loads of the round: the key row of lane c for the scores, value chunks for the sum ------------------
+        int tk = tb + c;
+        tk = tk < lo ? lo : (tk > p ? p : tk);                   // a row that exists; masked below
+        int row = a.rows_cap > 0 ? tk % a.rows_cap : tk;
+        const bf16_t* kp = a.k_pool + (((size_t)table[row / a.page] * a.KV + kvh) * a.page + row % a.page) * HD;
+        bf16x8 kf[KSTEPS];
 #pragma unroll
-        for (int jj = 0; jj < 2; jj++) {
-            const int tile = wave * 2 + jj;
-            const int tb = t0 + tile * 16;
-            f32x4 s = (f32x4){0.f, 0.f, 0.f, 0.f};
-            if (tb < t_end) {                        // wave-uniform
-                int tk = tb + c;
-                tk = tk < lo ? lo : (tk > p ? p : tk);           // a row that exists; masked below
-                const int row = a.rows_cap > 0 ? tk % a.rows_cap : tk;
-                const int pg = table[row / a.page];
-                const bf16_t* kp = a.k_pool + (((size_t)pg * a.KV + kvh) * a.page + row % a.page) * HD;
-                bf16x8 kf[KSTEPS];
-#pragma unroll
-                for (int ks = 0; ks < KSTEPS; ks++) {
-                    const int d0 = ks * 32 + g * 8;
-                    kf[ks] = ld_frag(kp + (d0 < HD ? d0 : 0), d0 < HD);
-                }
-#pragma unroll
-                for (int ks = 0; ks < KSTEPS; ks++) s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[ks], qf[ks], s, 0, 0, 0);
-            }
-            if (c < QT) {
-#pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const int kl = tile * 16 + g * 4 + i, tk = t0 + kl;
-                    const bool ok = tk >= lo && tk < t_end;
-                    s_lds[c][kl] = ok ? score_of(s[i], a.scale, a.cap) : -INFINITY;
-                }
-            }
+        for (int ks = 0; ks < KSTEPS; ks++) {
+            const int d0 = ks * 32 + g * 8;
+            kf[ks] = ld_frag(kp + (d0 < HD ? d0 : 0), d0 < HD);
         }
-        __syncthreads();
-        // ---- running softmax per query head: wave w takes heads w, w + 4, ... ---------------------------------
-        for (int qi = wave; qi < QT; qi += 4) {
-            const float v0 = s_lds[qi][lane], v1 = s_lds[qi][lane + 64];
-            const float mx = wave_max(fmaxf(v0, v1));
-            const float m_old = m_run[qi], m_new = fmaxf(m_old, mx);
-            float al = 1.f, p0 = 0.f, p1 = 0.f;
-            if (m_new != -INFINITY) {
-                al = __expf(m_old - m_new);
-                p0 = __expf(v0 - m_new);
-                p1 = __expf(v1 - m_new);
-            }
-            s_lds[qi][lane] = p0;
-            s_lds[qi][lane + 64] = p1;
-            const float sum = wave_sum(p0 + p1);
-            if (lane == 0) { m_run[qi] = m_new; l_run[qi] = l_run[qi] * al + sum; alpha_s[qi] = al; }
+        Frag vf[VPT];
+#pragma unroll
+        for (int j = 0; j < VPT; j++) {
+            const int kk = kgw + j * KGW;
+            int tv = tb + kk;
+            const bool on = pv_lane && kk < 16 && tv < t_end;
+            tv = tv < lo ? lo : (tv > p ? p : tv);
+            row = a.rows_cap > 0 ? tv % a.rows_cap : tv;
+            if (on) vf[j].u = *reinterpret_cast<const uint4*>(a.v_pool + (((size_t)table[row / a.page] * a.KV + kvh) * a.page + row % a.page) * HD + ch * 8);
+            else vf[j].u = make_uint4(0, 0, 0, 0);
         }
-        __syncthreads();
-        // ---- weighted sum of V: thread (chunk ch, key group kg) ------------------------------------------------
-        if (pv_thread) {
+        // ---- scores of 16 keys for the group's query heads: lane (c, g) gets keys g*4 .. g*4+3 of head c ----------
+        f32x4 s = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int qi = 0; qi < QT; qi++) {
-                const float al = alpha_s[qi];
+        for (int ks = 0; ks < KSTEPS; ks++) s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[ks], qf[ks], s, 0, 0, 0);
+        float mx = -INFINITY;
 #pragma unroll
-                for (int e = 0; e < 8; e++) acc[qi][e] *= al;
-            }
-            const int kmax = min(KB, t_end - t0);
-#pragma unroll 4
-            for (int kk = kg; kk < kmax; kk += KGROUPS) {
-                int tk = t0 + kk;
-                tk = tk < lo ? lo : tk;                          // hidden keys have probability 0
-                const int row = a.rows_cap > 0 ? tk % a.rows_cap : tk;
-                const int pg = table[row / a.page];
-                Frag vf;
-                vf.u = *reinterpret_cast<const uint4*>(a.v_pool + (((size_t)pg * a.KV + kvh) * a.page + row % a.page) * HD + ch * 8);
+        for (int i = 0; i < 4; i++) {
+            const int t = tb + g * 4 + i;
+            const bool ok = t >= lo && t < t_end;
+            s[i] = ok ? score_of(s[i], a.scale, a.cap) : -INFINITY;
+            mx = fmaxf(mx, s[i]);
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(m_run, mx);
+        float alpha = 1.f, psum = 0.f;
+        float pr[4] = {0.f, 0.f, 0.f, 0.f};
+        if (m_new != -INFINITY) {
+            alpha = __expf(m_run - m_new);
+#pragma unroll
+            for (int i = 0; i < 4; i++) { pr[i] = __expf(s[i] - m_new); psum += pr[i]; }
+        }
+        psum += __shfl_xor(psum, 16, 64);
+        psum += __shfl_xor(psum, 32, 64);
+        l_run = l_run * alpha + psum;
+        m_run = m_new;
+        if (c < QT) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) p_lds[wave][c][g * 4 + i] = pr[i];
+            if (g == 0) alpha_lds[wave][c] = alpha;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        // ---- weighted sum of the round's values -----------------------------------------------------------------------
+#pragma unroll
+        for (int qi = 0; qi < QT; qi++) {
+            const float al = alpha_lds[wave][qi];
+#pragma unroll
+            for (int e = 0; e < 8; e++) acc[qi][e] *= al;
+        }
+#pragma unroll
+        for (int j = 0; j < VPT; j++) {
+            const int kk = kgw + j * KGW;
+            if (kk < 16) {
                 float vv[8];
 #pragma unroll
-                for (int e = 0; e < 8; e++) vv[e] = bf16_to_f32(vf.h[e]);
+                for (int e = 0; e < 8; e++) vv[e] = bf16_to_f32(vf[j].h[e]);
 #pragma unroll
                 for (int qi = 0; qi < QT; qi++) {
-                    const float pr = s_lds[qi][kk];
+                    const float w = p_lds[wave][qi][kk];
 #pragma unroll
-                    for (int e = 0; e < 8; e++) acc[qi][e] = fmaf(pr, vv[e], acc[qi][e]);
+                    for (int e = 0; e < 8; e++) acc[qi][e] = fmaf(w, vv[e], acc[qi][e]);
                 }
             }
         }
-        __syncthreads();
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
     }
-    // ---- add the key groups' partial sums in group order and write ----------------------------------------------
+    // ---- the four waves' results: rescale to a common maximum, add in wave and key-group order, write -------------
+    if (c < QT && g == 0) { m_w[wave][c] = m_run; l_w[wave][c] = l_run; }
     for (int qi = 0; qi < QT; qi++) {
         if (qi >= G) break;
-        if (pv_thread) {
+        if (pv_lane) {
 #pragma unroll
-            for (int e = 0; e < 8; e++) red[kg * HD + ch * 8 + e] = acc[qi][e];
+            for (int e = 0; e < 8; e++) red[(wave * KGW + kgw) * HD + ch * 8 + e] = acc[qi][e];
         }
         __syncthreads();
         if (tid < HD) {
-            float sum = 0.f;
-            for (int k2 = 0; k2 < KGROUPS; k2++) sum += red[k2 * HD + tid];
+            float mx = -INFINITY;
+            for (int w = 0; w < 4; w++) mx = fmaxf(mx, m_w[w][qi]);
+            float num = 0.f, den = 0.f;
+            for (int w = 0; w < 4; w++) {
+                const float mw = m_w[w][qi];
+                if (mw == -INFINITY) continue;
+                const float f = __expf(mw - mx);
+                float part = 0.f;
+                for (int k2 = 0; k2 < KGW; k2++) part += red[(w * KGW + k2) * HD + tid];
+                num += f * part;
+                den += f * l_w[w][qi];
+            }
             const int head = kvh * G + qi;
             if (a.nsplit == 1) {
-                a.out[((size_t)seq * a.H + head) * HD + tid] = f32_to_bf16(sum / l_run[qi]);
+                a.out[((size_t)seq * a.H + head) * HD + tid] = f32_to_bf16(num / den);
             } else {
                 const size_t at = ((size_t)seq * a.H + head) * a.nsplit + split;
-                a.ws_o[at * HD + tid] = sum;
-                if (tid == 0) { a.ws_ml[at * 2] = m_run[qi]; a.ws_ml[at * 2 + 1] = l_run[qi]; }
+                a.ws_o[at * HD + tid] = num;
+                if (tid == 0) { a.ws_ml[at * 2] = mx; a.ws_ml[at * 2 + 1] = den; }
             }
         }
         __syncthreads();
@@ -400,11 +419,11 @@ extern "C" int tp_attn_decode(const void* q, long q_stride, int n_seq, int H, in
     }
     dim3 grid(KV, n_seq, nsplit);
     hipStream_t s = (hipStream_t)stream;
-    if (G <= 1) attn_decode_k<1><<<grid, 256, 0, s>>>(a);
-    else if (G <= 2) attn_decode_k<2><<<grid, 256, 0, s>>>(a);
-    else if (G <= 4) attn_decode_k<4><<<grid, 256, 0, s>>>(a);
-    else if (G <= 8) attn_decode_k<8><<<grid, 256, 0, s>>>(a);
-    else attn_decode_k<16><<<grid, 256, 0, s>>>(a);
+    if (G <= 1) attn_decode_k<1><<<grid, DTH, 0, s>>>(a);
+    else if (G <= 2) attn_decode_k<2><<<grid, DTH, 0, s>>>(a);
+    else if (G <= 4) attn_decode_k<4><<<grid, DTH, 0, s>>>(a);
+    else if (G <= 8) attn_decode_k<8><<<grid, DTH, 0, s>>>(a);
+    else attn_decode_k<16><<<grid, DTH, 0, s>>>(a);
     if (int rc = tp_check_launch("attention decode")) return rc;
     if (nsplit > 1) {
         attn_decode_combine_k<<<n_seq * H, HD < 64 ? 64 : HD, 0, s>>>(a.ws_o, a.ws_ml, nsplit, (bf16_t*)out);

@@ -43,8 +43,8 @@ __global__ void rms_norm_k(const TI* __restrict__ x, const float* __restrict__ g
 }
 
 // the same for rows of at most 256 * EPT elements: every element is read once and kept in registers
-template <typename TI, typename TO, int EPT>
-__global__ void __launch_bounds__(256)
+template <typename TI, typename TO, int EPT, int NTH>
+__global__ void __launch_bounds__(NTH)
 rms_norm_reg_k(const TI* __restrict__ x, const float* __restrict__ gain, float eps, TO* __restrict__ out, int D) {
     __shared__ float red[16];
     const TI* xr = x + (size_t)blockIdx.x * D;
@@ -53,7 +53,7 @@ rms_norm_reg_k(const TI* __restrict__ x, const float* __restrict__ gain, float e
     float ss = 0.f;
 #pragma unroll
     for (int j = 0; j < EPT; j++) {
-        const int i = threadIdx.x + j * 256;
+        const int i = threadIdx.x + j * NTH;
         v[j] = i < D ? ld_f32(xr + i) : 0.f;
         gn[j] = i < D ? gain[i] : 0.f;
     }
@@ -63,16 +63,18 @@ rms_norm_reg_k(const TI* __restrict__ x, const float* __restrict__ gain, float e
     const float scale = rsqrtf(ss / (float)D + eps);
 #pragma unroll
     for (int j = 0; j < EPT; j++) {
-        const int i = threadIdx.x + j * 256;
+        const int i = threadIdx.x + j * NTH;
         if (i < D) st_f32(orow + i, (v[j] * scale) * gn[j]);
     }
 }
 
 template <typename TI, typename TO>
 static void rms_norm_launch(const void* x, const float* gain, float eps, void* out, int M, int D, hipStream_t s) {
-    if (D <= 256 * 4) rms_norm_reg_k<TI, TO, 4><<<M, 256, 0, s>>>((const TI*)x, gain, eps, (TO*)out, D);
-    else if (D <= 256 * 12) rms_norm_reg_k<TI, TO, 12><<<M, 256, 0, s>>>((const TI*)x, gain, eps, (TO*)out, D);
-    else if (D <= 256 * 20) rms_norm_reg_k<TI, TO, 20><<<M, 256, 0, s>>>((const TI*)x, gain, eps, (TO*)out, D);
+    if (D <= 256 * 2) rms_norm_reg_k<TI, TO, 2, 256><<<M, 256, 0, s>>>((const TI*)x, gain, eps, (TO*)out, D);
+    else if (M <= 128 && D <= 1024 * 4) rms_norm_reg_k<TI, TO, 4, 1024><<<M, 1024, 0, s>>>((const TI*)x, gain, eps, (TO*)out, D);
+    else if (D <= 256 * 4) rms_norm_reg_k<TI, TO, 4, 256><<<M, 256, 0, s>>>((const TI*)x, gain, eps, (TO*)out, D);
+    else if (D <= 256 * 12) rms_norm_reg_k<TI, TO, 12, 256><<<M, 256, 0, s>>>((const TI*)x, gain, eps, (TO*)out, D);
+    else if (D <= 1024 * 8) rms_norm_reg_k<TI, TO, 8, 1024><<<M, 1024, 0, s>>>((const TI*)x, gain, eps, (TO*)out, D);
     else rms_norm_k<TI, TO><<<M, 256, 0, s>>>((const TI*)x, gain, eps, (TO*)out, D);
 }
 
@@ -122,8 +124,8 @@ __global__ void add_rms_norm_k(float* __restrict__ stream, const T* __restrict__
 
 // TR: type of the rows (float when they arrive as n_slices K slices of a product, each `slice_stride`
 // elements apart, added here in slice order); T: type of the normed output.
-template <typename TR, typename T, int EPT>
-__global__ void __launch_bounds__(256)
+template <typename TR, typename T, int EPT, int NTH>
+__global__ void __launch_bounds__(NTH)
 add_rms_norm_reg_k(float* __restrict__ stream, const TR* __restrict__ rows, int n_slices, long slice_stride,
                    const float* __restrict__ gain_post, float eps_post,
                    const float* __restrict__ gain_next, float eps_next, T* __restrict__ out, int D) {
@@ -133,7 +135,7 @@ add_rms_norm_reg_k(float* __restrict__ stream, const TR* __restrict__ rows, int 
     float a[EPT], v[EPT], gp[EPT], gn[EPT];
 #pragma unroll
     for (int j = 0; j < EPT; j++) {
-        const int i = threadIdx.x + j * 256;
+        const int i = threadIdx.x + j * NTH;
         const bool ok = i < D;
         a[j] = ok ? ld_f32(ar + i) : 0.f;
         for (int sl = 1; sl < n_slices; sl++) a[j] += ok ? ld_f32(ar + (size_t)sl * slice_stride + i) : 0.f;
@@ -152,7 +154,7 @@ add_rms_norm_reg_k(float* __restrict__ stream, const TR* __restrict__ rows, int 
     float ss2 = 0.f;
 #pragma unroll
     for (int j = 0; j < EPT; j++) {
-        const int i = threadIdx.x + j * 256;
+        const int i = threadIdx.x + j * NTH;
         float t = a[j];
         if (gain_post) t = (t * scale_a) * gp[j];
         v[j] += t;
@@ -164,7 +166,7 @@ add_rms_norm_reg_k(float* __restrict__ stream, const TR* __restrict__ rows, int 
     T* orow = out + (size_t)blockIdx.x * D;
 #pragma unroll
     for (int j = 0; j < EPT; j++) {
-        const int i = threadIdx.x + j * 256;
+        const int i = threadIdx.x + j * NTH;
         if (i < D) st_f32(orow + i, (v[j] * scale_s) * gn[j]);
     }
 }
@@ -172,11 +174,14 @@ add_rms_norm_reg_k(float* __restrict__ stream, const TR* __restrict__ rows, int 
 template <typename TR, typename T>
 static int add_rms_norm_launch(float* stream, const void* rows, int n_slices, long slice_stride, const float* gp, float ep,
                                const float* gn, float en, void* out, int M, int D, hipStream_t s) {
-    if (D <= 256 * 4) add_rms_norm_reg_k<TR, T, 4><<<M, 256, 0, s>>>(stream, (const TR*)rows, n_slices, slice_stride, gp, ep, gn, en, (T*)out, D);
-    else if (D <= 256 * 12) add_rms_norm_reg_k<TR, T, 12><<<M, 256, 0, s>>>(stream, (const TR*)rows, n_slices, slice_stride, gp, ep, gn, en, (T*)out, D);
-    else if (D <= 256 * 20) add_rms_norm_reg_k<TR, T, 20><<<M, 256, 0, s>>>(stream, (const TR*)rows, n_slices, slice_stride, gp, ep, gn, en, (T*)out, D);
+    // few rows: many threads per row (the kernel is bound by the latency of its loads, not by their volume)
+    if (D <= 256 * 2) add_rms_norm_reg_k<TR, T, 2, 256><<<M, 256, 0, s>>>(stream, (const TR*)rows, n_slices, slice_stride, gp, ep, gn, en, (T*)out, D);
+    else if (M <= 128 && D <= 1024 * 4) add_rms_norm_reg_k<TR, T, 4, 1024><<<M, 1024, 0, s>>>(stream, (const TR*)rows, n_slices, slice_stride, gp, ep, gn, en, (T*)out, D);
+    else if (D <= 256 * 4) add_rms_norm_reg_k<TR, T, 4, 256><<<M, 256, 0, s>>>(stream, (const TR*)rows, n_slices, slice_stride, gp, ep, gn, en, (T*)out, D);
+    else if (D <= 256 * 12) add_rms_norm_reg_k<TR, T, 12, 256><<<M, 256, 0, s>>>(stream, (const TR*)rows, n_slices, slice_stride, gp, ep, gn, en, (T*)out, D);
+    else if (D <= 1024 * 8) add_rms_norm_reg_k<TR, T, 8, 1024><<<M, 1024, 0, s>>>(stream, (const TR*)rows, n_slices, slice_stride, gp, ep, gn, en, (T*)out, D);
     else if (n_slices == 1 && sizeof(TR) == sizeof(T)) add_rms_norm_k<T><<<M, 256, 0, s>>>(stream, (const T*)rows, gp, ep, gn, en, (T*)out, D);
-    else return tp_fail("add_rms_norm: rows in slices need a width of at most %d, found %d", 256 * 20, D);
+    else return tp_fail("add_rms_norm: rows in slices need a width of at most %d, found %d", 1024 * 8, D);
     return 0;
 }
 
@@ -215,58 +220,59 @@ extern "C" int tp_gather_rows(const float* x, const int* rows, float* out, int n
 // Rotation: pair (d, d + rot/2), angle = pos * inv_freq[d], fp32 cos/sin (runtime/cuda/codebook_gemv.cu:219-230);
 // the cache keeps k after the rotation and v as projected (runtime/src/lib.rs:4487-4490).
 // A sequence's position p lives in row p (or p % rows_cap of a ring), found through its page list.
+// grid (rows, H + KV): block (r, j) rotates query head j, or for j >= H rotates key head j - H and writes it and
+// its value head into the cache straight from registers.
 template <typename T>
-__global__ void rope_kv_write_k(T* __restrict__ q, long q_stride, T* __restrict__ k, long k_stride,
-                                const T* __restrict__ v, long v_stride, int H, int KV, int hd,
-                                const float* __restrict__ inv_freq, int rot,
-                                const int* __restrict__ row_seq, const int* __restrict__ row_pos,
-                                const int* __restrict__ new_len, const int* __restrict__ table, int table_w,
-                                T* __restrict__ k_pool, T* __restrict__ v_pool, int page, int rows_cap) {
-    const int r = blockIdx.x;
+__global__ void __launch_bounds__(128)
+rope_kv_write_k(T* __restrict__ q, long q_stride, T* __restrict__ k, long k_stride,
+                const T* __restrict__ v, long v_stride, int H, int KV, int hd,
+                const float* __restrict__ inv_freq, int rot,
+                const int* __restrict__ row_seq, const int* __restrict__ row_pos,
+                const int* __restrict__ new_len, const int* __restrict__ table, int table_w,
+                T* __restrict__ k_pool, T* __restrict__ v_pool, int page, int rows_cap) {
+    const int r = blockIdx.x, j = blockIdx.y;
     const int pos = row_pos[r];
     const int half = rot / 2;
-    if (half > 0) {
-        T* qr = q + (size_t)r * q_stride;
-        for (int i = threadIdx.x; i < H * half; i += blockDim.x) {
-            const int h = i / half, d = i % half;
-            const float ang = (float)pos * inv_freq[d];
-            const float c = cosf(ang), s = sinf(ang);
-            T* a = qr + h * hd + d;
-            const float x0 = ld_f32(a), x1 = ld_f32(a + half);
-            st_f32(a, x0 * c - x1 * s);
-            st_f32(a + half, x1 * c + x0 * s);
+    const bool is_q = j < H;
+    if (!is_q && !k) return;
+    T* x = is_q ? q + (size_t)r * q_stride + (size_t)j * hd : k + (size_t)r * k_stride + (size_t)(j - H) * hd;
+    T* kdst = nullptr;
+    T* vdst = nullptr;
+    const T* vsrc = nullptr;
+    if (!is_q) {
+        const int seq = row_seq[r];
+        int row = pos;
+        bool keep = true;
+        if (rows_cap > 0) {
+            keep = pos + rows_cap >= new_len[seq];       // else a later row of this step takes the same ring row
+            row = pos % rows_cap;
+        }
+        const int pg = keep ? table[(size_t)seq * table_w + row / page] : -1;
+        if (pg >= 0) {
+            const size_t off = (((size_t)pg * KV + (j - H)) * page + row % page) * hd;
+            kdst = k_pool + off;
+            vdst = v_pool + off;
+            vsrc = v + (size_t)r * v_stride + (size_t)(j - H) * hd;
         }
     }
-    if (!k) return;
-    T* kr = k + (size_t)r * k_stride;
-    if (half > 0) {
-        for (int i = threadIdx.x; i < KV * half; i += blockDim.x) {
-            const int h = i / half, d = i % half;
-            const float ang = (float)pos * inv_freq[d];
-            const float c = cosf(ang), s = sinf(ang);
-            T* a = kr + h * hd + d;
-            const float x0 = ld_f32(a), x1 = ld_f32(a + half);
-            st_f32(a, x0 * c - x1 * s);
-            st_f32(a + half, x1 * c + x0 * s);
+    for (int f = threadIdx.x; f < half; f += blockDim.x) {     // one thread per pair (f, f + half)
+        const float ang = (float)pos * inv_freq[f];
+        const float c = cosf(ang), sn = sinf(ang);
+        const float x0 = ld_f32(x + f), x1 = ld_f32(x + f + half);
+        st_f32(x + f, x0 * c - x1 * sn);
+        st_f32(x + f + half, x1 * c + x0 * sn);
+        if (kdst) {
+            st_f32(kdst + f, x0 * c - x1 * sn);
+            st_f32(kdst + f + half, x1 * c + x0 * sn);
+            vdst[f] = vsrc[f];
+            vdst[f + half] = vsrc[f + half];
         }
     }
-    const int seq = row_seq[r];
-    int row = pos;
-    if (rows_cap > 0) {
-        if (pos + rows_cap < new_len[seq]) return;      // a later row of this step takes the same ring row
-        row = pos % rows_cap;
-    }
-    const int pg = table[(size_t)seq * table_w + row / page];
-    if (pg < 0) return;
-    __syncthreads();                                      // the rotated k of this row is read back below
-    const T* vr = v + (size_t)r * v_stride;
-    const int in_page = row % page;
-    for (int i = threadIdx.x; i < KV * hd; i += blockDim.x) {
-        const int h = i / hd, d = i % hd;
-        const size_t dst = (((size_t)pg * KV + h) * page + in_page) * hd + d;
-        k_pool[dst] = kr[i];
-        v_pool[dst] = vr[i];
-    }
+    if (kdst)
+        for (int d = rot + threadIdx.x; d < hd; d += blockDim.x) {   // elements outside the rotation
+            kdst[d] = x[d];
+            vdst[d] = vsrc[d];
+        }
 }
 
 extern "C" int tp_rope_kv_write(void* q, long q_stride, void* k, long k_stride, const void* v, long v_stride,
@@ -281,11 +287,14 @@ extern "C" int tp_rope_kv_write(void* q, long q_stride, void* k, long k_stride, 
                "rope_kv_write: keys without values, cache pools or page table");
     TP_REQUIRE(rows_cap >= 0 && (rows_cap == 0 || rows_cap % page == 0), "rope_kv_write: ring of %d rows is no multiple of the page size %d", rows_cap, page);
     hipStream_t s = (hipStream_t)stream;
+    TP_REQUIRE(H + KV <= 65535, "rope_kv_write: %d heads exceed one launch", H + KV);
+    dim3 grid(M, H + (k ? KV : 0));
+    const int threads = hd <= 64 ? 64 : 128;
     if (dtype == TP_BF16)
-        rope_kv_write_k<bf16_t><<<M, 256, 0, s>>>((bf16_t*)q, q_stride, (bf16_t*)k, k_stride, (const bf16_t*)v, v_stride, H, KV, hd,
+        rope_kv_write_k<bf16_t><<<grid, threads, 0, s>>>((bf16_t*)q, q_stride, (bf16_t*)k, k_stride, (const bf16_t*)v, v_stride, H, KV, hd,
             inv_freq, rot, row_seq, row_pos, new_len, table, table_w, (bf16_t*)k_pool, (bf16_t*)v_pool, page, rows_cap);
     else if (dtype == TP_F32)
-        rope_kv_write_k<float><<<M, 256, 0, s>>>((float*)q, q_stride, (float*)k, k_stride, (const float*)v, v_stride, H, KV, hd,
+        rope_kv_write_k<float><<<grid, threads, 0, s>>>((float*)q, q_stride, (float*)k, k_stride, (const float*)v, v_stride, H, KV, hd,
             inv_freq, rot, row_seq, row_pos, new_len, table, table_w, (float*)k_pool, (float*)v_pool, page, rows_cap);
     else return tp_fail("rope_kv_write: unknown dtype %d", dtype);
     return tp_check_launch("rope_kv_write");

@@ -30,10 +30,75 @@ argmax_k(const float* __restrict__ logits, int V, int* __restrict__ out) {
     }
 }
 
-extern "C" int tp_argmax(const float* logits, int B, int V, int* out, void* stream) {
+// stage 1 of the two-stage form: grid (parts, rows), each block scans one contiguous part of a row
+__global__ void __launch_bounds__(256)
+argmax_part_k(const float* __restrict__ logits, int V, int per_part, float* __restrict__ pval, int* __restrict__ pidx) {
+    __shared__ float sval[4];
+    __shared__ int sidx[4];
+    const float* z = logits + (size_t)blockIdx.y * V;
+    const int lo = blockIdx.x * per_part, hi = min(V, lo + per_part);
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int i = lo + threadIdx.x; i < hi; i += blockDim.x) {
+        const float v = z[i];
+        if (v > bv || (v == bv && i < bi)) { bv = v; bi = i; }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(bv, o, 64);
+        const int oi = __shfl_xor(bi, o, 64);
+        if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+    }
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (lane == 0) { sval[wave] = bv; sidx[wave] = bi; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < 4; w++)
+            if (sval[w] > bv || (sval[w] == bv && sidx[w] < bi)) { bv = sval[w]; bi = sidx[w]; }
+        pval[blockIdx.y * gridDim.x + blockIdx.x] = bv;
+        pidx[blockIdx.y * gridDim.x + blockIdx.x] = bi;
+    }
+}
+
+// stage 2: one wave per row over the parts' winners
+__global__ void __launch_bounds__(64)
+argmax_final_k(const float* __restrict__ pval, const int* __restrict__ pidx, int parts, int* __restrict__ out) {
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int i = threadIdx.x; i < parts; i += 64) {
+        const float v = pval[blockIdx.x * parts + i];
+        const int id = pidx[blockIdx.x * parts + i];
+        if (v > bv || (v == bv && id < bi)) { bv = v; bi = id; }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(bv, o, 64);
+        const int oi = __shfl_xor(bi, o, 64);
+        if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+    }
+    if (threadIdx.x == 0) out[blockIdx.x] = bi == 0x7fffffff ? 0 : bi;
+}
+
+extern "C" long tp_argmax_workspace_bytes(int B, int V) {
+    const int parts = V >= 16384 ? 64 : 1;
+    return parts > 1 ? (long)B * parts * 8 : 0;
+}
+
+extern "C" int tp_argmax(const float* logits, int B, int V, int* out, void* workspace, void* stream) {
     TP_REQUIRE(B > 0 && V > 0, "argmax: empty shape B=%d V=%d", B, V);
-    argmax_k<<<B, 1024, 0, (hipStream_t)stream>>>(logits, V, out);
-    return tp_check_launch("argmax");
+    TP_REQUIRE(B <= 65535, "argmax: %d rows exceed one launch", B);
+    const int parts = V >= 16384 ? 64 : 1;
+    hipStream_t s = (hipStream_t)stream;
+    if (parts == 1 || !workspace) {
+        argmax_k<<<B, 1024, 0, s>>>(logits, V, out);
+        return tp_check_launch("argmax");
+    }
+    float* pval = (float*)workspace;
+    int* pidx = (int*)(pval + (size_t)B * parts);
+    argmax_part_k<<<dim3(parts, B), 256, 0, s>>>(logits, V, tp_cdiv(V, parts), pval, pidx);
+    if (int rc = tp_check_launch("argmax (parts)")) return rc;
+    argmax_final_k<<<B, 64, 0, s>>>(pval, pidx, parts, out);
+    return tp_check_launch("argmax (final)");
 }
 
 // ---- repetition penalty: every distinct recent token once, z / penalty if z > 0 else z * penalty

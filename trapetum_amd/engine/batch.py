@@ -55,10 +55,11 @@ class StaticStep:
 
     RING = 8
 
-    def __init__(self, rt, cache, n_seq):
+    def __init__(self, rt, cache, n_seq, length_bound):
         import torch
         self.rt = rt
         self.n_seq = n_seq
+        self.length_bound = length_bound        # the graph serves steps whose sequences are no longer than this
         self.table_widths = [g.max_pages_per_seq for g in cache.kv_groups]
         size = 6 * n_seq + 1 + sum(n_seq * w for w in self.table_widths)
         self.size = size
@@ -132,10 +133,10 @@ class StepContext:
 
     def max_keys(self, site):
         """Most keys any sequence of this step can see at this cache site (a host number, for launch geometry).
-        With fixed step memory (a captured graph) it is the most the cache allows."""
-        if self.static is not None:
-            return site.rows_cap or self.cache.max_context
+        With fixed step memory (a captured graph) it is the graph's bound on the lengths."""
         longest = max(s + c for s, c in zip(self.starts, self.counts))
+        if self.static is not None:
+            longest = max(longest, self.static.length_bound)
         return min(longest, site.rows_cap) if site.rows_cap else longest
 
     # keys and values of this step, for entries that read another entry's cache during a prefill

@@ -1,4 +1,4 @@
-"""Decode steps replayed from captured HIP graphs, one graph per batch size.
+"""Decode steps replayed from captured HIP graphs, one graph per batch size and bound on the lengths.
 
 A decode step is some three hundred small launches; replaying them from a graph removes the host's share of
 the step (the reference reports the same lever for its own loop: runtime/README.md:49-58, and wraps capture
@@ -32,11 +32,18 @@ class GraphedDecode:
         counts, starts, want, tok = model.prepare(cache, slots, tokens)
         if any(c != 1 for c in counts):
             raise ValueError("graphed steps take one token per sequence")
-        b = len(slots)
+        # launch geometry that depends on lengths (how many blocks share a sequence's keys) is fixed in a
+        # graph, so a graph serves lengths up to a bound: the next power of two, at least 1024
+        longest = max(s + 1 for s in starts)
+        bound = 1024
+        while bound < longest:
+            bound *= 2
+        bound = min(bound, cache.max_context)
+        b = (len(slots), bound)
         cap = self.by_batch.get(b)
         if cap is None:
-            static = StaticStep(model.rt, cache, b)
-            tokens_static = torch.zeros(b, dtype=torch.int32, device=model.rt.device)
+            static = StaticStep(model.rt, cache, len(slots), bound)
+            tokens_static = torch.zeros(len(slots), dtype=torch.int32, device=model.rt.device)
             tokens_static.copy_(tok)
             ctx = StepContext(model.rt, cache, slots, counts, starts, want, static=static)
             logits = model.run(ctx, tokens_static)          # this step, eagerly; also loads what capture must not

@@ -23,7 +23,8 @@ _CORE_SIGS = {
     "tp_linear": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P, _L, _I, _I, _P],
     "tp_attn_simple_prefill": [_P, _L, _P, _L, _P, _L, _I, _I, _I, _I, _I, _P, _P, _P, _F, _F, _I, _P, _P],
     "tp_attn_simple_decode": [_P, _L, _I, _I, _I, _I, _I, _P, _P, _I, _P, _P, _I, _I, _F, _F, _I, _P, _P],
-    "tp_argmax": [_P, _I, _I, _P, _P],
+    "tp_argmax": [_P, _I, _I, _P, _P, _P],
+    "tp_argmax_workspace_bytes": [_I, _I],
     "tp_repetition_penalty": [_P, _I, _I, _P, _I, _F, _P],
     "tp_sample": [_P, _I, _I, _F, _I, _F, _P, _P, _P],
 }
@@ -305,7 +306,8 @@ class HipOps:
         if self._fast_attention(q.dtype, H, KV, hd) and k_pool.shape[2] % 16 == 0:
             lib = self.attn_lib(hd)
             keys = int(max_keys) if max_keys else k_pool.shape[0] * k_pool.shape[2]
-            nsplit = max(1, min(-(-512 // (n * KV)), -(-keys // 128), 64))
+            # enough blocks to fill the chip, each with at least one round of 64 keys
+            nsplit = max(1, min(-(-768 // (n * KV)), -(-keys // 64), 128))
             floats = lib.tp_attn_decode_workspace_floats(n, H, nsplit)
             ws = torch.empty(floats, dtype=torch.float32, device=self.device) if floats else None
             self._call(lib, "tp_attn_decode", q.data_ptr(), qs, n, H, KV, new_len.data_ptr(), table.data_ptr(),
@@ -324,7 +326,10 @@ class HipOps:
         if logits.dtype != torch.float32 or logits.dim() != 2 or not logits.is_contiguous():
             raise KernelError("argmax: logits must be contiguous float32 [rows, vocab]")
         out = torch.empty(logits.shape[0], dtype=torch.int32, device=self.device)
-        self._call(self.lib, "tp_argmax", logits.data_ptr(), logits.shape[0], logits.shape[1], out.data_ptr(), self._stream())
+        nbytes = self.lib.tp_argmax_workspace_bytes(logits.shape[0], logits.shape[1])
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=self.device) if nbytes else None
+        self._call(self.lib, "tp_argmax", logits.data_ptr(), logits.shape[0], logits.shape[1], out.data_ptr(),
+                   ws.data_ptr() if ws is not None else None, self._stream())
         return out
 
     def apply_repetition_penalty(self, logits, recent, penalty):
