@@ -35,10 +35,18 @@ __device__ __forceinline__ bf16x8 ld_frag(const bf16_t* p, bool ok) {
     else f.u = make_uint4(0, 0, 0, 0);
     return f.v;
 }
-__device__ __forceinline__ float score_of(float dot, float scale, float cap) {
-    float s = dot * scale;
-    if (cap > 0.f) s = cap * tanhf(s / cap);
-    return s;
+// tanh through one exponential and one reciprocal: 1 - 2 / (1 + e^(2x)); exact at both ends, relative error of a
+// few 1e-7 elsewhere (the scores are rounded to bf16 probabilities afterwards)
+__device__ __forceinline__ float tanh_fast(float x) {
+    return 1.f - 2.f * __builtin_amdgcn_rcpf(1.f + __expf(2.f * x));
+}
+// scale_over_cap = scale / cap, so that a capped score costs two multiplications around the tanh
+__device__ __forceinline__ float score_of(float dot, float scale, float cap, float scale_over_cap) {
+    return cap > 0.f ? cap * tanh_fast(dot * scale_over_cap) : dot * scale;
+}
+__device__ __forceinline__ bf16_t bf16_bits(float f) {
+    __bf16 b = (__bf16)f;                          // one conversion instruction on gfx950, round to nearest even
+    return __builtin_bit_cast(bf16_t, b);
 }
 }  // namespace
 
@@ -51,6 +59,7 @@ __device__ __forceinline__ float score_of(float dot, float scale, float cap) {
 struct PrefillArgs {
     const bf16_t* q; long q_stride; const bf16_t* k; long k_stride; const bf16_t* v; long v_stride;
     int H, KV; const int* cu_rows; float scale, cap; int window; bf16_t* out;
+    const bf16_t* vt; long vt_rows;      // V transposed: [kv head][head element][padded key slot], vt_rows slots per row
 };
 
 namespace {
@@ -59,12 +68,46 @@ constexpr int KLD = HDP + 8;                    // LDS row strides in elements: 
 constexpr int VLD = BKV + 8;
 }
 
+// V of the step, transposed once per layer so that the attention blocks copy it into LDS as it lies:
+// vt[kv head][d][slot], a sequence's keys in groups of 32 slots (its region padded to a multiple of 32), the keys
+// of a group permuted as the second product's operand wants them (key a*16 + g*4 + b at slot g*8 + a*4 + b).
+__device__ __forceinline__ int vt_base_of(const int* cu_rows, int seq) {
+    int base = 0;
+    for (int s = 0; s < seq; s++) base += (cu_rows[s + 1] - cu_rows[s] + BKV - 1) / BKV * BKV;
+    return base;
+}
+
+__global__ void __launch_bounds__(256)
+v_transpose_k(const bf16_t* __restrict__ v, long v_stride, int KV, const int* __restrict__ cu_rows,
+              bf16_t* __restrict__ vt, long vt_rows) {
+    __shared__ bf16_t tile[BKV][HD + 2];
+    const int seq = blockIdx.z, kvh = blockIdx.y, kt = blockIdx.x * BKV;
+    const int row0 = cu_rows[seq], T = cu_rows[seq + 1] - row0;
+    if (kt >= T) return;
+    const int base = vt_base_of(cu_rows, seq) + kt;
+    for (int i = threadIdx.x; i < BKV * NCH; i += 256) {
+        const int key = i / NCH, ch = i % NCH;
+        Frag f;
+        f.u = make_uint4(0, 0, 0, 0);
+        if (kt + key < T) f.u = *reinterpret_cast<const uint4*>(v + (size_t)(row0 + kt + key) * v_stride + (size_t)kvh * HD + ch * 8);
+#pragma unroll
+        for (int e = 0; e < 8; e++) tile[key][ch * 8 + e] = f.h[e];
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < HD * BKV; i += 256) {          // consecutive threads: consecutive slots of one d
+        const int d = i / BKV, slot = i % BKV;
+        const int key = ((slot >> 2) & 1) * 16 + (slot >> 3) * 4 + (slot & 3);   // slot g*8 + a*4 + b holds key a*16 + g*4 + b
+        vt[((size_t)kvh * HD + d) * vt_rows + base + slot] = tile[key][d];
+    }
+}
+
 __global__ void __launch_bounds__(256)
 attn_prefill_k(PrefillArgs a) {
     __shared__ __attribute__((aligned(16))) bf16_t Ks[BKV * KLD];
     __shared__ __attribute__((aligned(16))) bf16_t Vt[HD * VLD];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = lane & 15, g = lane >> 4;
-    const int seq = blockIdx.z, h = blockIdx.y, q0 = blockIdx.x * 64;
+    // late query tiles see the most keys: they are given the low block ids, which start first
+    const int seq = blockIdx.z, h = blockIdx.y, q0 = (gridDim.x - 1 - blockIdx.x) * 64;
     const int row0 = a.cu_rows[seq], T = a.cu_rows[seq + 1] - row0;
     if (q0 >= T) return;
     const int kvh = h / (a.H / a.KV);
@@ -84,28 +127,53 @@ attn_prefill_k(PrefillArgs a) {
 #pragma unroll
     for (int dt = 0; dt < HD / 16; dt++) o[dt] = (f32x4){0.f, 0.f, 0.f, 0.f};
     float m_i = -INFINITY, l_i = 0.f;
+    const float soc = a.cap > 0.f ? a.scale / a.cap : 0.f;
 
     int k_lo = a.window > 0 ? max(0, q0 - a.window + 1) : 0;
     k_lo &= ~(BKV - 1);
     const int k_hi = min(T, q0 + 64);
-    for (int kt = k_lo; kt < k_hi; kt += BKV) {
-        __syncthreads();
-        for (int i = tid; i < BKV * NCH; i += 256) {
-            const int key = i / NCH, ch = i % NCH, tk = kt + key;
-            Frag kf, vf;
-            if (tk < T) {
-                kf.u = *reinterpret_cast<const uint4*>(a.k + (size_t)(row0 + tk) * a.k_stride + (size_t)kvh * HD + ch * 8);
-                vf.u = *reinterpret_cast<const uint4*>(a.v + (size_t)(row0 + tk) * a.v_stride + (size_t)kvh * HD + ch * 8);
-            } else {
-                kf.u = make_uint4(0, 0, 0, 0);
-                vf.u = make_uint4(0, 0, 0, 0);
-            }
-            *reinterpret_cast<uint4*>(Ks + key * KLD + ch * 8) = kf.u;
-            const int pos = ((key & 15) >> 2) * 8 + (key >> 4) * 4 + (key & 3);      // key = a*16 + g*4 + b -> g*8 + a*4 + b
+    // a tile's rows travel global memory -> registers (one tile ahead, while the tile before is being used) -> LDS;
+    // K as stored, V from its transposed copy: HD rows of 32 slots (64 bytes) each
+    constexpr int KTASKS = (BKV * NCH + 255) / 256;                 // (key, 16-byte chunk) per thread
+    constexpr int VTASKS = (HD * 4 + 255) / 256;                    // (head element, 16-byte chunk of its 32 slots)
+    Frag fk[KTASKS], fv[VTASKS];
+    const int vbase = vt_base_of(a.cu_rows, seq);
+    auto fetch = [&](int kt) {
 #pragma unroll
-            for (int e = 0; e < 8; e++) Vt[(ch * 8 + e) * VLD + pos] = vf.h[e];
+        for (int t = 0; t < KTASKS; t++) {
+            const int i = tid + t * 256;
+            const int key = i / NCH, ch = i % NCH, tk = kt + key;
+            fk[t].u = make_uint4(0, 0, 0, 0);
+            if (i < BKV * NCH && tk < T)
+                fk[t].u = *reinterpret_cast<const uint4*>(a.k + (size_t)(row0 + tk) * a.k_stride + (size_t)kvh * HD + ch * 8);
         }
+#pragma unroll
+        for (int t = 0; t < VTASKS; t++) {
+            const int i = tid + t * 256;
+            const int d = i >> 2, part = i & 3;
+            fv[t].u = make_uint4(0, 0, 0, 0);
+            if (i < HD * 4)
+                fv[t].u = *reinterpret_cast<const uint4*>(a.vt + ((size_t)kvh * HD + d) * a.vt_rows + vbase + kt + part * 8);
+        }
+    };
+    auto stage = [&]() {
+#pragma unroll
+        for (int t = 0; t < KTASKS; t++) {
+            const int i = tid + t * 256;
+            if (i < BKV * NCH) *reinterpret_cast<uint4*>(Ks + (i / NCH) * KLD + (i % NCH) * 8) = fk[t].u;
+        }
+#pragma unroll
+        for (int t = 0; t < VTASKS; t++) {
+            const int i = tid + t * 256;
+            if (i < HD * 4) *reinterpret_cast<uint4*>(Vt + (i >> 2) * VLD + (i & 3) * 8) = fv[t].u;
+        }
+    };
+    fetch(k_lo);
+    for (int kt = k_lo; kt < k_hi; kt += BKV) {
+        __syncthreads();                             // the tile before has been used by every wave
+        stage();
         __syncthreads();
+        if (kt + BKV < k_hi) fetch(kt + BKV);
         const bool visible = qw0 < T && kt <= qw0 + 15 && !(a.window > 0 && kt + BKV - 1 < qw0 - a.window + 1);
         if (!visible) continue;                      // wave-uniform: every key of the tile is hidden from the wave's queries
 
@@ -121,14 +189,19 @@ attn_prefill_k(PrefillArgs a) {
             }
         }
         // lane holds the scores of keys kt + j*16 + g*4 + i for its query qpos
+        // a tile every query of the wave sees whole needs no mask (wave-uniform)
+        const bool whole = kt + BKV - 1 <= qw0 && qw0 + 15 < T && (a.window <= 0 || qw0 + 15 - kt < a.window);
         float mx = -INFINITY;
 #pragma unroll
         for (int j = 0; j < 2; j++)
 #pragma unroll
             for (int i = 0; i < 4; i++) {
-                const int tk = kt + j * 16 + g * 4 + i;
-                const bool ok = tk <= qpos && tk < T && (a.window <= 0 || qpos - tk < a.window);
-                const float v = ok ? score_of(s[j][i], a.scale, a.cap) : -INFINITY;
+                float v = score_of(s[j][i], a.scale, a.cap, soc);
+                if (!whole) {
+                    const int tk = kt + j * 16 + g * 4 + i;
+                    const bool ok = tk <= qpos && tk < T && (a.window <= 0 || qpos - tk < a.window);
+                    v = ok ? v : -INFINITY;
+                }
                 s[j][i] = v;
                 mx = fmaxf(mx, v);
             }
@@ -147,18 +220,19 @@ attn_prefill_k(PrefillArgs a) {
                 for (int i = 0; i < 4; i++) {
                     const float p = __expf(s[j][i] - m_new);
                     sum += p;
-                    pf.h[j * 4 + i] = f32_to_bf16(p);
+                    pf.h[j * 4 + i] = bf16_bits(p);
                 }
         }
         sum += __shfl_xor(sum, 16, 64);
         sum += __shfl_xor(sum, 32, 64);
         l_i = l_i * alpha + sum;
         m_i = m_new;
+        const bool rescale = __any(alpha != 1.f);              // once the running maxima settle, nothing to rescale
 #pragma unroll
         for (int dt = 0; dt < HD / 16; dt++) {
             Frag vf;
             vf.u = *reinterpret_cast<const uint4*>(Vt + (dt * 16 + c) * VLD + g * 8);
-            o[dt] = o[dt] * alpha;
+            if (rescale) o[dt] = o[dt] * alpha;
             o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf.v, o[dt], 0, 0, 0);
         }
     }
@@ -168,22 +242,33 @@ attn_prefill_k(PrefillArgs a) {
 #pragma unroll
     for (int dt = 0; dt < HD / 16; dt++) {
         ushort4 pk;
-        pk.x = f32_to_bf16(o[dt][0] * inv); pk.y = f32_to_bf16(o[dt][1] * inv);
-        pk.z = f32_to_bf16(o[dt][2] * inv); pk.w = f32_to_bf16(o[dt][3] * inv);
+        pk.x = bf16_bits(o[dt][0] * inv); pk.y = bf16_bits(o[dt][1] * inv);
+        pk.z = bf16_bits(o[dt][2] * inv); pk.w = bf16_bits(o[dt][3] * inv);
         *reinterpret_cast<ushort4*>(orow + dt * 16 + g * 4) = pk;
     }
 }
 
+// elements of the transposed copy of V the prefill kernel needs as workspace
+extern "C" long tp_attn_prefill_workspace_elems(int M, int KV, int n_seq) {
+    return (long)KV * HD * ((long)M + (long)BKV * n_seq + BKV);
+}
+
 extern "C" int tp_attn_prefill(const void* q, long q_stride, const void* k, long k_stride, const void* v, long v_stride,
                                int M, int H, int KV, const int* cu_rows, int n_seq, int max_count,
-                               float scale, float cap, int window, void* out, void* stream) {
+                               float scale, float cap, int window, void* out, void* workspace, void* stream) {
     TP_REQUIRE(M > 0 && H > 0 && KV > 0 && n_seq > 0 && max_count > 0, "attention prefill: empty shape");
     TP_REQUIRE(H % KV == 0, "attention: %d query heads are no multiple of %d kv heads", H, KV);
     TP_REQUIRE(q_stride % 8 == 0 && k_stride % 8 == 0 && v_stride % 8 == 0 && (uintptr_t)q % 16 == 0 &&
                (uintptr_t)k % 16 == 0 && (uintptr_t)v % 16 == 0, "attention prefill: rows must be 16-byte aligned");
     TP_REQUIRE(H <= 65535 && n_seq <= 65535, "attention prefill: %d heads / %d sequences exceed one launch", H, n_seq);
+    TP_REQUIRE(workspace && (uintptr_t)workspace % 16 == 0, "attention prefill: needs its 16-byte aligned workspace");
+    TP_REQUIRE(KV <= 65535, "attention prefill: %d kv heads exceed one launch", KV);
+    const long vt_rows = (long)M + (long)BKV * n_seq + BKV;         // every sequence's region is padded to whole groups
+    v_transpose_k<<<dim3(tp_cdiv(max_count, BKV), KV, n_seq), 256, 0, (hipStream_t)stream>>>(
+        (const bf16_t*)v, v_stride, KV, cu_rows, (bf16_t*)workspace, vt_rows);
+    if (int rc = tp_check_launch("attention prefill (transpose of V)")) return rc;
     PrefillArgs a{(const bf16_t*)q, q_stride, (const bf16_t*)k, k_stride, (const bf16_t*)v, v_stride, H, KV, cu_rows,
-                  scale, cap, window, (bf16_t*)out};
+                  scale, cap, window, (bf16_t*)out, (const bf16_t*)workspace, vt_rows};
     dim3 grid(tp_cdiv(max_count, 64), H, n_seq);
     attn_prefill_k<<<grid, 256, 0, (hipStream_t)stream>>>(a);
     return tp_check_launch("attention prefill");
@@ -256,6 +341,7 @@ attn_decode_k(DecodeArgs a) {
 #pragma unroll
         for (int e = 0; e < 8; e++) acc[qi][e] = 0.f;
     float m_run = -INFINITY, l_run = 0.f;            // of query head c, over this wave's keys so far
+    const float soc = a.cap > 0.f ? a.scale / a.cap : 0.f;
 
     for (int tb = t_begin + wave * 16; tb < t_end; tb += ROUND) {
         // ---- loads of the round: the key row of lane c for the scores, value chunks for the sum ------------------
@@ -289,7 +375,7 @@ attn_decode_k(DecodeArgs a) {
         for (int i = 0; i < 4; i++) {
             const int t = tb + g * 4 + i;
             const bool ok = t >= lo && t < t_end;
-            s[i] = ok ? score_of(s[i], a.scale, a.cap) : -INFINITY;
+            s[i] = ok ? score_of(s[i], a.scale, a.cap, soc) : -INFINITY;
             mx = fmaxf(mx, s[i]);
         }
         mx = fmaxf(mx, __shfl_xor(mx, 16, 64));

@@ -90,20 +90,25 @@ static int check_args(const GemmArgs& a) {
     return 0;
 }
 
-// algo: 0 = choose, 1 = plain, 2 = skinny matrix-core, 3 = tiled matrix-core
+// algo: 0 = choose, 1 = plain, 2 = skinny matrix-core, 3 = tiled matrix-core, 4 = tiled with direct loads
 static int pick(const GemmArgs& a, int algo) {
     if (algo == 1) return 1;
     if (algo == 2) return gemm_skinny_supports(a) ? 2 : -2;
     if (algo == 3) return gemm_mfma_supports(a) ? 3 : -3;
+    if (algo == 4) return gemm_tiled_supports(a) ? 4 : -4;
     if (gemm_skinny_supports(a)) return 2;
     if (gemm_mfma_supports(a)) return 3;
     return 1;
 }
 
-extern "C" long tp_linear_workspace_bytes(int in_dtype, int out_dtype, int M, int N, int K, int epilogue, int units, int algo) {
-    GemmArgs a{nullptr, nullptr, nullptr, in_dtype, out_dtype, M, N, K, epilogue, 1.f, units, nullptr, 0, 0, nullptr};
+// bytes of workspace a product needs; with defer, a positive multiple of M * N * 4 above one slice means the
+// product comes back as that many K slices
+extern "C" long tp_linear_workspace_bytes(int in_dtype, int out_dtype, int M, int N, int K, int epilogue, int units,
+                                          int defer, int algo) {
+    GemmArgs a{nullptr, nullptr, nullptr, in_dtype, out_dtype, M, N, K, epilogue, 1.f, units, nullptr, 0, defer, nullptr};
     const int p = pick(a, algo);
     if (p == 2) return (long)gemm_skinny_workspace(a);
+    if (p == 3) { const int s = gemm_mfma_splits(a); return s > 1 ? (long)s * M * N * 4 : 0; }
     if (p == 1 && epilogue == TP_EPI_GATED) return (long)M * N * 4;
     return 0;
 }
@@ -118,5 +123,6 @@ extern "C" int tp_linear(const void* x, const void* w, void* y, int in_dtype, in
     TP_REQUIRE(p > 0, "linear: the requested kernel (%d) does not take M=%d N=%d K=%d dtype %d", algo, M, N, K, in_dtype);
     if (p == 2) return gemm_skinny_launch(a);
     if (p == 3) return gemm_mfma_launch(a);
+    if (p == 4) return gemm_tiled_launch(a);
     return gemm_simple_launch(a);
 }

@@ -22,12 +22,16 @@ union Frag { uint4 u; bf16x8 v; };
 template <int EPI>
 __global__ void __launch_bounds__(256)
 gemm_mfma_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __restrict__ Y,
-            int M, int N, int K, int m_tiles, int out_dtype, float cap, int units) {
+            int M, int N, int K, int m_tiles, int out_dtype, float cap, int units, int k_per_split) {
     __shared__ __attribute__((aligned(16))) bf16_t As[BM * LDS];
     __shared__ __attribute__((aligned(16))) bf16_t Bs[BN * LDS];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 15, g = lane >> 4;
     const int wm = wave >> 1, wn = wave & 1;
     const int m0 = (blockIdx.x % m_tiles) * BM, n0 = (blockIdx.x / m_tiles) * BN;
+    // a K slice per blockIdx.y: slices go to Y as float32 [slices, M, N] for the consumer to add in slice order
+    const int k_begin = blockIdx.y * k_per_split;
+    const int k_end = min(K, k_begin + k_per_split);
+    if (gridDim.y > 1) Y = (float*)Y + (size_t)blockIdx.y * M * N;
 
     // global -> register staging: 4 chunks of 16 bytes per thread and operand; chunk c: row c / 8, k chunk c % 8
     uint4 ra[4], rb[4];
@@ -37,8 +41,8 @@ gemm_mfma_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __
             const int c = tid + i * 256, row = c >> 3, kc = (c & 7) * 8;
             const int k = k0 + kc;
             const int m = m0 + row, n = n0 + row;
-            ra[i] = (m < M && k < K) ? *reinterpret_cast<const uint4*>(X + (size_t)m * K + k) : make_uint4(0, 0, 0, 0);
-            rb[i] = (n < N && k < K) ? *reinterpret_cast<const uint4*>(W + (size_t)n * K + k) : make_uint4(0, 0, 0, 0);
+            ra[i] = (m < M && k < k_end) ? *reinterpret_cast<const uint4*>(X + (size_t)m * K + k) : make_uint4(0, 0, 0, 0);
+            rb[i] = (n < N && k < k_end) ? *reinterpret_cast<const uint4*>(W + (size_t)n * K + k) : make_uint4(0, 0, 0, 0);
         }
     };
     auto stage = [&]() {
@@ -56,12 +60,12 @@ gemm_mfma_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __
 #pragma unroll
         for (int j = 0; j < 4; j++) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
-    fetch(0);
-    for (int k0 = 0; k0 < K; k0 += BK) {
+    fetch(k_begin);
+    for (int k0 = k_begin; k0 < k_end; k0 += BK) {
         __syncthreads();                       // everyone is done reading the previous tile
         stage();
         __syncthreads();
-        if (k0 + BK < K) fetch(k0 + BK);
+        if (k0 + BK < k_end) fetch(k0 + BK);
 #pragma unroll
         for (int ks = 0; ks < BK; ks += 32) {
             Frag a[4], b[4];
@@ -114,6 +118,17 @@ bool gemm_mfma_supports(const GemmArgs& a) {
     return a.in_dtype == TP_BF16 && a.K % 8 == 0;
 }
 
+// K slices for products whose tiles alone do not fill the chip and whose consumer adds the slices (defer)
+int gemm_mfma_splits(const GemmArgs& a) {
+    if (!a.defer || a.epilogue != TP_EPI_NONE) return 1;
+    const long blocks = (long)tp_cdiv(a.M, BM) * tp_cdiv(a.N, BN);
+    if (blocks >= 200 || a.K < 1024) return 1;         // measured: no gain at 288 tiles and more
+    int s = (int)(640 / blocks);
+    if (s > a.K / 512) s = a.K / 512;
+    if (s > 4) s = 4;
+    return s < 1 ? 1 : s;
+}
+
 int gemm_mfma_launch(const GemmArgs& a) {
     TP_REQUIRE(gemm_mfma_supports(a), "tiled product: needs bf16 and K a multiple of 8 (K=%d)", a.K);
     TP_REQUIRE(((uintptr_t)a.x % 16 == 0) && ((uintptr_t)a.w % 16 == 0), "tiled product: operands must be 16-byte aligned");
@@ -122,11 +137,20 @@ int gemm_mfma_launch(const GemmArgs& a) {
     TP_REQUIRE(blocks < (1L << 31), "tiled product: %ld tiles are too many for one launch", blocks);
     const bf16_t* x = (const bf16_t*)a.x;
     const bf16_t* w = (const bf16_t*)a.w;
+    const int splits = gemm_mfma_splits(a);
+    if (splits > 1) {
+        const size_t need = (size_t)splits * a.M * a.N * sizeof(float);
+        TP_REQUIRE(a.workspace && a.workspace_bytes >= need, "tiled product: workspace of %zu bytes, %zu needed", a.workspace_bytes, need);
+        const int kps = tp_cdiv(tp_cdiv(a.K, splits), BK) * BK;
+        dim3 grid((unsigned)blocks, tp_cdiv(a.K, kps));
+        gemm_mfma_k<TP_EPI_NONE><<<grid, 256, 0, a.stream>>>(x, w, a.workspace, a.M, a.N, a.K, m_tiles, TP_F32, 0.f, 0, kps);
+        return tp_check_launch("linear (tiled kernel, K slices)");
+    }
     if (a.epilogue == TP_EPI_GATED)
-        gemm_mfma_k<TP_EPI_GATED><<<(unsigned)blocks, 256, 0, a.stream>>>(x, w, a.y, a.M, a.N, a.K, m_tiles, a.out_dtype, a.cap, a.units);
+        gemm_mfma_k<TP_EPI_GATED><<<(unsigned)blocks, 256, 0, a.stream>>>(x, w, a.y, a.M, a.N, a.K, m_tiles, a.out_dtype, a.cap, a.units, a.K);
     else if (a.epilogue == TP_EPI_SOFTCAP)
-        gemm_mfma_k<TP_EPI_SOFTCAP><<<(unsigned)blocks, 256, 0, a.stream>>>(x, w, a.y, a.M, a.N, a.K, m_tiles, a.out_dtype, a.cap, a.units);
+        gemm_mfma_k<TP_EPI_SOFTCAP><<<(unsigned)blocks, 256, 0, a.stream>>>(x, w, a.y, a.M, a.N, a.K, m_tiles, a.out_dtype, a.cap, a.units, a.K);
     else
-        gemm_mfma_k<TP_EPI_NONE><<<(unsigned)blocks, 256, 0, a.stream>>>(x, w, a.y, a.M, a.N, a.K, m_tiles, a.out_dtype, a.cap, a.units);
+        gemm_mfma_k<TP_EPI_NONE><<<(unsigned)blocks, 256, 0, a.stream>>>(x, w, a.y, a.M, a.N, a.K, m_tiles, a.out_dtype, a.cap, a.units, a.K);
     return tp_check_launch("linear (tiled kernel)");
 }

@@ -21,6 +21,7 @@ _CORE_SIGS = {
     "tp_rope_kv_write": [_P, _L, _P, _L, _P, _L, _I, _I, _I, _I, _I, _P, _I, _P, _P, _P, _P, _I, _P, _P, _I, _I, _P],
     "tp_gated_act": [_P, _P, _I, _I, _I, _P],
     "tp_linear": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P, _L, _I, _I, _P],
+    "tp_linear_workspace_bytes": [_I, _I, _I, _I, _I, _I, _I, _I, _I],
     "tp_attn_simple_prefill": [_P, _L, _P, _L, _P, _L, _I, _I, _I, _I, _I, _P, _P, _P, _F, _F, _I, _P, _P],
     "tp_attn_simple_decode": [_P, _L, _I, _I, _I, _I, _I, _P, _P, _I, _P, _P, _I, _I, _F, _F, _I, _P, _P],
     "tp_argmax": [_P, _I, _I, _P, _P, _P],
@@ -29,7 +30,8 @@ _CORE_SIGS = {
     "tp_sample": [_P, _I, _I, _F, _I, _F, _P, _P, _P],
 }
 _ATTN_SIGS = {
-    "tp_attn_prefill": [_P, _L, _P, _L, _P, _L, _I, _I, _I, _P, _I, _I, _F, _F, _I, _P, _P],
+    "tp_attn_prefill": [_P, _L, _P, _L, _P, _L, _I, _I, _I, _P, _I, _I, _F, _F, _I, _P, _P, _P],
+    "tp_attn_prefill_workspace_elems": [_I, _I, _I],
     "tp_attn_decode": [_P, _L, _I, _I, _I, _P, _P, _I, _P, _P, _I, _I, _F, _F, _I, _P, _P, _I, _P],
     "tp_attn_decode_workspace_floats": [_I, _I, _I],
 }
@@ -65,7 +67,7 @@ def _bind(lib, sigs):
     for name, args in sigs.items():
         fn = getattr(lib, name)
         fn.argtypes = args
-        fn.restype = _c.c_long if name.endswith("_bytes") or name.endswith("_floats") else _I
+        fn.restype = _c.c_long if name.endswith(("_bytes", "_floats", "_elems")) else _I
 
 
 class HipOps:
@@ -235,7 +237,8 @@ class HipOps:
             raise KernelError(f"linear: rows have {k} columns, the matrix {w.shape[1]}")
         cols = units if epilogue == EPI_GATED else n
         algo = self.force_linear
-        nbytes = self.lib.tp_linear_workspace_bytes(_code(x.dtype), _code(out_dtype), m, n, k, epilogue, units, algo)
+        nbytes = self.lib.tp_linear_workspace_bytes(_code(x.dtype), _code(out_dtype), m, n, k, epilogue, units,
+                                                    1 if defer else 0, algo)
         if defer and epilogue == EPI_NONE and nbytes and nbytes % (m * n * 4) == 0 and nbytes // (m * n * 4) > 1:
             slices = torch.empty((nbytes // (m * n * 4), m, n), dtype=torch.float32, device=self.device)
             self._call(self.lib, "tp_linear", x.data_ptr(), w.data_ptr(), None, _code(x.dtype), _code(out_dtype),
@@ -277,9 +280,11 @@ class HipOps:
         n_seq = cu_rows.numel() - 1
         out = torch.empty((m, H * hd), dtype=out_dtype, device=self.device)
         if self._fast_attention(q.dtype, H, KV, hd):
-            self._call(self.attn_lib(hd), "tp_attn_prefill", q.data_ptr(), qs, k.data_ptr(), ks, v.data_ptr(), vs,
+            lib = self.attn_lib(hd)
+            ws = torch.empty(lib.tp_attn_prefill_workspace_elems(m, KV, n_seq), dtype=torch.bfloat16, device=self.device)
+            self._call(lib, "tp_attn_prefill", q.data_ptr(), qs, k.data_ptr(), ks, v.data_ptr(), vs,
                        m, H, KV, cu_rows.data_ptr(), n_seq, int(max_count), float(scale), float(softcap), int(window),
-                       out.data_ptr(), self._stream())
+                       out.data_ptr(), ws.data_ptr(), self._stream())
             return out
         if row_seq is None:
             counts = (cu_rows[1:] - cu_rows[:-1]).long()
