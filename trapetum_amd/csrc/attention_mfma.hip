@@ -292,6 +292,10 @@ struct DecodeArgs {
 };
 
 namespace {
+// In the decode kernel a lane's two loads of a pair of product steps are adjacent 16-byte pieces, so the four lanes
+// of a key row fetch a whole 128-byte line per pair: step ks, lane group g -> head elements dofs .. dofs + 7.
+constexpr int DSTEPS = 2 * ((HD + 63) / 64);
+__device__ __forceinline__ int dofs(int ks, int g) { return (ks >> 1) * 64 + g * 16 + (ks & 1) * 8; }
 constexpr int DTH = 256;                         // 4 waves; each scores and sums its own 16 keys of a round
 constexpr int ROUND = 64;                        // keys a block takes per round
 constexpr int KGW = 64 / NCH > 16 ? 16 : 64 / NCH;   // key groups of a wave: lanes with one chunk index walk the keys KGW apart
@@ -324,11 +328,25 @@ attn_decode_k(DecodeArgs a) {
         return;
     }
     const int* table = a.table + (size_t)seq * a.table_w;
+    // Where the 16 keys of a tile live.  Tiles start at multiples of 16 positions; position t is row t, or row
+    // t % rows_cap of a ring (rows_cap a multiple of the page size, the page size a power of two >= 16), so a tile
+    // lies in one page, in 16 consecutive rows: one page-table entry per tile, looked up once for the wave.
+    const int page_shift = __ffs(a.page) - 1, page_mask = a.page - 1;
+    const int ring_lo = a.rows_cap > 0 ? lo_al % a.rows_cap : 0;
+    auto tile_offset = [&](int tb) -> size_t {                     // element offset of the tile's first row in a pool
+        int row = tb;
+        if (a.rows_cap > 0) {
+            row = ring_lo + (tb - lo_al);
+            row = row >= a.rows_cap ? row - a.rows_cap : row;
+        }
+        const int pg = table[row >> page_shift];
+        return (((size_t)pg * a.KV + kvh) * a.page + (row & page_mask)) * HD;
+    };
 
-    bf16x8 qf[KSTEPS];
+    bf16x8 qf[DSTEPS];
 #pragma unroll
-    for (int ks = 0; ks < KSTEPS; ks++) {
-        const int d0 = ks * 32 + g * 8;
+    for (int ks = 0; ks < DSTEPS; ks++) {
+        const int d0 = dofs(ks, g);
         const bool ok = c < G && d0 < HD;
         qf[ks] = ld_frag(a.q + (size_t)seq * a.q_stride + (size_t)(kvh * G + (ok ? c : 0)) * HD + (ok ? d0 : 0), ok);
     }
@@ -345,31 +363,29 @@ attn_decode_k(DecodeArgs a) {
 
     for (int tb = t_begin + wave * 16; tb < t_end; tb += ROUND) {
         // ---- loads of the round: the key row of lane c for the scores, value chunks for the sum ------------------
+        const size_t tile = tile_offset(__builtin_amdgcn_readfirstlane(tb));
         int tk = tb + c;
         tk = tk < lo ? lo : (tk > p ? p : tk);                   // a row that exists; masked below
-        int row = a.rows_cap > 0 ? tk % a.rows_cap : tk;
-        const bf16_t* kp = a.k_pool + (((size_t)table[row / a.page] * a.KV + kvh) * a.page + row % a.page) * HD;
-        bf16x8 kf[KSTEPS];
+        const bf16_t* kp = a.k_pool + tile + (size_t)(tk - tb) * HD;
+        bf16x8 kf[DSTEPS];
 #pragma unroll
-        for (int ks = 0; ks < KSTEPS; ks++) {
-            const int d0 = ks * 32 + g * 8;
+        for (int ks = 0; ks < DSTEPS; ks++) {
+            const int d0 = dofs(ks, g);
             kf[ks] = ld_frag(kp + (d0 < HD ? d0 : 0), d0 < HD);
         }
         Frag vf[VPT];
 #pragma unroll
-        for (int j = 0; j < VPT; j++) {
-            const int kk = kgw + j * KGW;
+        for (int j = 0; j < VPT; j++) {              // unconditional loads of rows that exist: a hidden or surplus
+            int kk = kgw + j * KGW;                  // key gets probability 0 (or is skipped) in the sum below
+            kk = kk > 15 ? 15 : kk;
             int tv = tb + kk;
-            const bool on = pv_lane && kk < 16 && tv < t_end;
             tv = tv < lo ? lo : (tv > p ? p : tv);
-            row = a.rows_cap > 0 ? tv % a.rows_cap : tv;
-            if (on) vf[j].u = *reinterpret_cast<const uint4*>(a.v_pool + (((size_t)table[row / a.page] * a.KV + kvh) * a.page + row % a.page) * HD + ch * 8);
-            else vf[j].u = make_uint4(0, 0, 0, 0);
+            vf[j].u = *reinterpret_cast<const uint4*>(a.v_pool + tile + (size_t)(tv - tb) * HD + ch * 8);
         }
         // ---- scores of 16 keys for the group's query heads: lane (c, g) gets keys g*4 .. g*4+3 of head c ----------
         f32x4 s = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int ks = 0; ks < KSTEPS; ks++) s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[ks], qf[ks], s, 0, 0, 0);
+        for (int ks = 0; ks < DSTEPS; ks++) s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[ks], qf[ks], s, 0, 0, 0);
         float mx = -INFINITY;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
@@ -492,7 +508,8 @@ extern "C" int tp_attn_decode(const void* q, long q_stride, int n_seq, int H, in
     TP_REQUIRE(H % KV == 0, "attention: %d query heads are no multiple of %d kv heads", H, KV);
     const int G = H / KV;
     TP_REQUIRE(G <= 16, "attention decode (matrix-core kernel): %d query heads per kv head exceed 16", G);
-    TP_REQUIRE(page > 0 && page % 16 == 0 && table_w > 0, "attention decode: page size %d must be a positive multiple of 16", page);
+    TP_REQUIRE(page >= 16 && (page & (page - 1)) == 0 && table_w > 0, "attention decode (matrix-core kernel): page size %d must be a power of two, at least 16", page);
+    TP_REQUIRE(rows_cap == 0 || window <= rows_cap, "attention decode: a window of %d keys does not fit a ring of %d rows", window, rows_cap);
     TP_REQUIRE(rows_cap >= 0 && rows_cap % page == 0, "attention decode: ring of %d rows is no multiple of the page size %d", rows_cap, page);
     TP_REQUIRE(nsplit >= 1 && (nsplit == 1 || workspace), "attention decode: %d slices need a workspace", nsplit);
     TP_REQUIRE(q_stride % 8 == 0 && (uintptr_t)q % 16 == 0, "attention decode: query rows must be 16-byte aligned");

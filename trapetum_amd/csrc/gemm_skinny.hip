@@ -63,18 +63,35 @@ gemm_skinny_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* 
 #pragma unroll
         for (int b = 0; b < MT; b++) acc[a][b] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
-    constexpr int U = 4;                                  // rounds in flight
-    for (int kw = kbeg + wave * 32; kw < kend; kw += 128 * U) {
-        bf16x8 a[U][NT], b[U][MT];
+    // Two register sets of U rounds each: while one set feeds the products, the loads of the next U rounds are
+    // in flight.  Loads are unconditional (a branch around a load would make the compiler wait for it at the
+    // join): past the end of the slice they read the slice's last chunk and X's fragment is zeroed instead.
+    constexpr int U = MT >= 4 ? 2 : 4;
+    union FragU { uint4 u; bf16x8 v; };
+    const int klast = kend - 8;
+    auto load = [&](int kw, bf16x8 (&a)[U][NT], bf16x8 (&b)[U][MT]) {
 #pragma unroll
         for (int u = 0; u < U; u++) {
             const int k = kw + u * 128 + g * 8;
             const bool ok = k < kend;
+            const int kc = ok ? k : klast;
 #pragma unroll
-            for (int t = 0; t < NT; t++) a[u][t] = load_frag(wrow[t] + k, ok);
+            for (int t = 0; t < NT; t++) {
+                FragU f;
+                f.u = *reinterpret_cast<const uint4*>(wrow[t] + kc);
+                a[u][t] = f.v;
+            }
 #pragma unroll
-            for (int t = 0; t < MT; t++) b[u][t] = load_frag(xrow[t] + k, ok && xok[t]);
+            for (int t = 0; t < MT; t++) {
+                FragU f;
+                f.u = *reinterpret_cast<const uint4*>(xrow[t] + kc);
+                const uint32_t keep = (uint32_t) - (int)(ok && xok[t]);      // all ones or zero: an AND, not a branch
+                f.u.x &= keep; f.u.y &= keep; f.u.z &= keep; f.u.w &= keep;
+                b[u][t] = f.v;
+            }
         }
+    };
+    auto mma = [&](bf16x8 (&a)[U][NT], bf16x8 (&b)[U][MT]) {
 #pragma unroll
         for (int u = 0; u < U; u++)
 #pragma unroll
@@ -82,6 +99,21 @@ gemm_skinny_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* 
 #pragma unroll
                 for (int t = 0; t < MT; t++)
                     acc[s][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][s], b[u][t], acc[s][t], 0, 0, 0);
+    };
+    bf16x8 a0[U][NT], b0[U][MT], a1[U][NT], b1[U][MT];
+    int kw = kbeg + wave * 32;
+    if (kw < kend) {
+        load(kw, a0, b0);
+        while (true) {
+            load(kw + 128 * U, a1, b1);
+            mma(a0, b0);
+            kw += 128 * U;
+            if (kw >= kend) break;
+            load(kw + 128 * U, a0, b0);
+            mma(a1, b1);
+            kw += 128 * U;
+            if (kw >= kend) break;
+        }
     }
 
 #pragma unroll

@@ -308,7 +308,8 @@ class HipOps:
         if table.dtype != torch.int32 or table.dim() != 2 or table.shape[0] != n or not table.is_contiguous():
             raise KernelError("attention_decode: the page table must be contiguous int32 [sequences, pages]")
         out = torch.empty((n, H * hd), dtype=out_dtype, device=self.device)
-        if self._fast_attention(q.dtype, H, KV, hd) and k_pool.shape[2] % 16 == 0:
+        page = k_pool.shape[2]
+        if self._fast_attention(q.dtype, H, KV, hd) and page >= 16 and page & (page - 1) == 0:
             lib = self.attn_lib(hd)
             keys = int(max_keys) if max_keys else k_pool.shape[0] * k_pool.shape[2]
             # enough blocks to fill the chip, each with at least one round of 64 keys
