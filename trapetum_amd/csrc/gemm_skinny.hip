@@ -28,13 +28,13 @@ __device__ __forceinline__ void store_out(void* y, int out_dtype, size_t idx, fl
     else ((bf16_t*)y)[idx] = f32_to_bf16(v);
 }
 
-// MT: 16-row tiles of X (rows padded to 16 * MT); NT: 16-row tiles of W per block (2 for a gated product:
-// the gate tile and the up tile of the same 16 units).
+// MT: 16-row tiles of X (rows padded to 16 * MT); NT: 16-row tiles of W per block, all fed by the same X
+// fragments (a gated product needs an even number: gate tile and up tile of the same 16 units alternate).
 template <int MT, int NT>
 __global__ void __launch_bounds__(256)
 gemm_skinny_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __restrict__ Y, float* __restrict__ part,
               int M, int N, int K, int k_per_split, int n_splits, int out_dtype, int epilogue, float cap, int units) {
-    __shared__ float red[4][NT][MT][64][4];
+    __shared__ float red[4][MT][64][4];                   // one W tile's partial tiles of the four waves at a time
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
     const int n0 = blockIdx.x * (16 * NT);
     const int split = blockIdx.y;
@@ -116,41 +116,46 @@ gemm_skinny_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* 
         }
     }
 
-#pragma unroll
-    for (int s = 0; s < NT; s++)
-#pragma unroll
-        for (int t = 0; t < MT; t++)
-#pragma unroll
-            for (int i = 0; i < 4; i++) red[wave][s][t][lane][i] = acc[s][t][i];
-    __syncthreads();
-
     // thread -> one element of every tile: lane l2 = tid / 4, component i = tid % 4
     const int l2 = threadIdx.x >> 2, i = threadIdx.x & 3;
     const int nl = (l2 >> 4) * 4 + i;                     // W row within the tile
     const int ml = l2 & 15;                               // X row within the tile
+    float v[MT][NT];
+#pragma unroll
+    for (int s = 0; s < NT; s++) {                        // the waves' partial tiles are added in wave order
+        if (s > 0) __syncthreads();
+#pragma unroll
+        for (int t = 0; t < MT; t++)
+#pragma unroll
+            for (int c = 0; c < 4; c++) red[wave][t][lane][c] = acc[s][t][c];
+        __syncthreads();
+#pragma unroll
+        for (int t = 0; t < MT; t++)
+            v[t][s] = ((red[0][t][l2][i] + red[1][t][l2][i]) + red[2][t][l2][i]) + red[3][t][l2][i];
+    }
+
 #pragma unroll
     for (int t = 0; t < MT; t++) {
         const int m = t * 16 + ml;
-        float v[NT];
-#pragma unroll
-        for (int s = 0; s < NT; s++)
-            v[s] = ((red[0][s][t][l2][i] + red[1][s][t][l2][i]) + red[2][s][t][l2][i]) + red[3][s][t][l2][i];
         if (m >= M) continue;
         if (n_splits > 1) {
 #pragma unroll
             for (int s = 0; s < NT; s++) {
                 const int n = n0 + s * 16 + nl;
-                if (n < N) part[((size_t)split * M + m) * N + n] = v[s];
+                if (n < N) part[((size_t)split * M + m) * N + n] = v[t][s];
             }
-        } else if (NT == 2 && epilogue == TP_EPI_GATED) {
-            const int unit = (n0 >> 1) + nl;
-            if (unit < units) store_out(Y, out_dtype, (size_t)m * units + unit, gelu_tanh_f(v[0]) * v[NT - 1]);
+        } else if (NT >= 2 && epilogue == TP_EPI_GATED) {
+#pragma unroll
+            for (int s = 0; s + 1 < NT; s += 2) {         // tiles alternate: 16 gate rows, the 16 up rows of the same units
+                const int unit = ((n0 + s * 16) >> 1) + nl;
+                if (unit < units) store_out(Y, out_dtype, (size_t)m * units + unit, gelu_tanh_f(v[t][s]) * v[t][s + 1]);
+            }
         } else {
 #pragma unroll
             for (int s = 0; s < NT; s++) {
                 const int n = n0 + s * 16 + nl;
                 if (n >= N) continue;
-                float o = v[s];
+                float o = v[t][s];
                 if (epilogue == TP_EPI_SOFTCAP) o = softcap_f(o, cap);
                 store_out(Y, out_dtype, (size_t)m * N + n, o);
             }
@@ -188,7 +193,17 @@ bool gemm_skinny_supports(const GemmArgs& a) {
 }
 
 static void plan(const GemmArgs& a, int& nt, int& blocks, int& splits, int& k_per_split) {
-    nt = a.epilogue == TP_EPI_GATED ? 2 : 1;
+    // W tiles per block: every tile reuses the block's X fragments, so more tiles mean less X traffic per byte
+    // of W (which matters from 16 rows on), as long as tiles x K slices still fill the chip
+    const int gated = a.epilogue == TP_EPI_GATED;
+    const int kslices = a.K / 512 > 1 ? a.K / 512 : 1;
+    nt = gated ? 2 : 1;
+    if (a.M > 16) {
+        if ((long)tp_cdiv(a.N, 64) * kslices >= 512) nt = 4;
+        else if ((long)tp_cdiv(a.N, 32) * kslices >= 512) nt = 2;
+    } else if (a.N >= 65536) {
+        nt = 2;
+    }
     blocks = tp_cdiv(a.N, 16 * nt);
     int want = tp_cdiv(512, blocks);
     int most = a.K / 512;
@@ -207,7 +222,10 @@ size_t gemm_skinny_workspace(const GemmArgs& a) {
 
 template <int MT>
 static void launch_mt(const GemmArgs& a, int nt, dim3 grid, float* part, int kps, int splits) {
-    if (nt == 2)
+    if (nt == 4)
+        gemm_skinny_k<MT, 4><<<grid, 256, 0, a.stream>>>((const bf16_t*)a.x, (const bf16_t*)a.w, a.y, part, a.M, a.N, a.K,
+                                                         kps, splits, a.out_dtype, a.epilogue, a.cap, a.units);
+    else if (nt == 2)
         gemm_skinny_k<MT, 2><<<grid, 256, 0, a.stream>>>((const bf16_t*)a.x, (const bf16_t*)a.w, a.y, part, a.M, a.N, a.K,
                                                          kps, splits, a.out_dtype, a.epilogue, a.cap, a.units);
     else
