@@ -136,6 +136,30 @@ def attention_decode(q, H, KV, hd, new_len, table, k_pool, v_pool, rows_cap, sca
     return out.to(out_dtype)
 
 
+def fuses_decode_step(dtype, H, KV, hd, k_pool):
+    return False
+
+
+def attention_decode_step(qkv, H, KV, hd, inv_freq, rotary_dim, new_len, table, k_pool, v_pool, rows_cap, scale, softcap,
+                          window, out_dtype, max_keys=None, write_kv=True, splits=None):
+    """The fused decode step as its three parts: qkv float32 [n, (H + 2 KV) hd] (already summed over K slices),
+    rotated in float32 and rounded once to the cache's dtype."""
+    n = qkv.shape[0]
+    pos = new_len.to(torch.int32) - 1
+    q = _rotate(qkv[:, :H * hd].float().reshape(n, H, hd), pos, inv_freq, rotary_dim).reshape(n, H * hd).to(k_pool.dtype)
+    if write_kv:
+        k = _rotate(qkv[:, H * hd:(H + KV) * hd].float().reshape(n, KV, hd), pos, inv_freq, rotary_dim).to(k_pool.dtype)
+        v = qkv[:, (H + KV) * hd:].reshape(n, KV, hd).to(k_pool.dtype)
+        page = k_pool.shape[2]
+        for i in range(n):
+            row = int(pos[i]) % rows_cap if rows_cap else int(pos[i])
+            pg = int(table[i, row // page])
+            assert pg >= 0
+            k_pool[pg, :, row % page, :] = k[i]
+            v_pool[pg, :, row % page, :] = v[i]
+    return attention_decode(q, H, KV, hd, new_len, table, k_pool, v_pool, rows_cap, scale, softcap, window, out_dtype)
+
+
 def rows(r, dtype):
     return r
 

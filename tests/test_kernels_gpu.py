@@ -250,9 +250,65 @@ def test_attention_decode(ops, plain, dt, H, KV, hd, lens, page, window, rows_ca
         got = ops.attention_decode(qlast.to(DEV), H, KV, hd, c["new_len"].to(DEV), c["table"].to(DEV),
                                    pools_ref[0].to(DEV), pools_ref[1].to(DEV), rows_cap, scale, cap, window, DT[dt],
                                    max_keys=max(lens))
+        if not plain:
+            for splits in (1, 2, 5):
+                again = ops.attention_decode(qlast.to(DEV), H, KV, hd, c["new_len"].to(DEV), c["table"].to(DEV),
+                                             pools_ref[0].to(DEV), pools_ref[1].to(DEV), rows_cap, scale, cap, window,
+                                             DT[dt], max_keys=max(lens), splits=splits)
+                assert rel_l2(again, ref) < 8e-3, splits
     finally:
         ops.force_plain_attention = False
     assert rel_l2(got, ref) < (3e-6 if dt == "f32" else 8e-3)
+
+
+@pytest.mark.parametrize("splits", [None, 1, 3])
+@pytest.mark.parametrize("slices", [0, 1, 3])
+@pytest.mark.parametrize("H,KV,hd,lens,page,window,rows_cap,cap", ATTN_CASES)
+def test_attention_decode_step(ops, splits, slices, H, KV, hd, lens, page, window, rows_cap, cap):
+    """Rotation, cache write and attention of a decode step in one launch, against the three reference parts.  The
+    cache holds every earlier position; the step's projections come as bf16 rows (slices 0) or as float32 K slices."""
+    from trapetum_amd.kernels.ops import SplitRows
+    n_pages, n = 24, len(lens)
+    c = build_cache_case(torch.bfloat16, H, KV, hd, lens, page, rows_cap, n_pages, 70)
+    rot = hd if hd != 80 else 48                            # one case with a rotation over part of the head
+    inv_freq = c["inv_freq"][:rot // 2].contiguous()
+    pools_ref = [torch.full((n_pages, KV, page, hd), 7.0, dtype=torch.bfloat16) for _ in range(2)]
+    earlier = c["row_pos"] < (c["new_len"][c["row_seq"].long()] - 1)          # all rows but each sequence's last
+    keep = earlier.nonzero().flatten()
+    ref_ops.rope_kv_write(c["q"].cpu()[keep].clone(), c["k"].cpu()[keep].clone(), c["v"].cpu()[keep], H, KV, hd, inv_freq, rot,
+                          c["row_seq"][keep], c["row_pos"][keep], c["new_len"] - 1, c["table"], pools_ref[0], pools_ref[1], rows_cap)
+    pools = [p.to(DEV) for p in pools_ref]
+    last = torch.tensor([int(c["cu"][i + 1]) - 1 for i in range(n)])
+    qkv = torch.cat([c["q"].cpu()[last], c["k"].cpu()[last], c["v"].cpu()[last]], dim=1).float()
+    if slices:
+        parts = torch.randn(slices, *qkv.shape, generator=torch.Generator().manual_seed(71))
+        parts[0] += qkv - parts.sum(0)
+        given, summed = SplitRows(parts.contiguous().to(DEV)), parts[0].clone()
+        for sl in range(1, slices):
+            summed += parts[sl]
+    else:
+        given, summed = qkv.to(torch.bfloat16).to(DEV), qkv.to(torch.bfloat16).float()
+    scale = 1.0 / math.sqrt(hd * 1.3)
+    ref = ref_ops.attention_decode_step(summed, H, KV, hd, inv_freq, rot, c["new_len"], c["table"], pools_ref[0], pools_ref[1],
+                                        rows_cap, scale, cap, window, torch.float32)
+    if not ops.fuses_decode_step(torch.bfloat16, H, KV, hd, pools[0]):
+        assert H // KV > 16
+        pytest.skip("more than 16 query heads per kv head run on the separate kernels")
+    got = ops.attention_decode_step(given, H, KV, hd, inv_freq.to(DEV), rot, c["new_len"].to(DEV), c["table"].to(DEV),
+                                    pools[0], pools[1], rows_cap, scale, cap, window, torch.bfloat16, max_keys=max(lens),
+                                    splits=splits)
+    assert rel_l2(got, ref) < 8e-3
+    assert rel_l2(pools[0], pools_ref[0]) < 6e-3 and rel_l2(pools[1], pools_ref[1]) < 6e-3
+    assert torch.equal((pools[0].cpu() != 7.0).any(dim=-1), (pools_ref[0] != 7.0).any(dim=-1))      # no other row touched
+    # queries only, on a cache that another run filled: the pools stay as they are
+    before = [p.clone() for p in pools]
+    got_q = ops.attention_decode_step(given.slices[..., :H * hd].contiguous() if slices else given[:, :H * hd].contiguous(),
+                                      H, KV, hd, inv_freq.to(DEV), rot, c["new_len"].to(DEV), c["table"].to(DEV),
+                                      pools[0], pools[1], rows_cap, scale, cap, window, torch.bfloat16, max_keys=max(lens),
+                                      write_kv=False, splits=splits) if not slices else None
+    if got_q is not None:
+        assert rel_l2(got_q, ref) < 8e-3
+        assert torch.equal(before[0], pools[0]) and torch.equal(before[1], pools[1])
 
 
 def test_attention_far_key_stands_out(ops):
@@ -273,7 +329,8 @@ def test_attention_far_key_stands_out(ops):
             ops.force_plain_attention = plain
             try:
                 got = ops.attention_decode(qb.to(DEV), H, KV, hd, c["new_len"].to(DEV), c["table"].to(DEV),
-                                           pools[0].to(DEV), pools[1].to(DEV), 0, 1.0, 0.0, 0, torch.bfloat16, max_keys=n)
+                                           pools[0].to(DEV), pools[1].to(DEV), 0, 1.0, 0.0, 0, torch.bfloat16, max_keys=n,
+                                           splits=None if plain else 1 + target % 7)
             finally:
                 ops.force_plain_attention = False
             want = c["v"].cpu().float().reshape(n, KV, hd)[target].repeat_interleave(H // KV, dim=0).reshape(1, H * hd)

@@ -287,8 +287,12 @@ extern "C" int tp_attn_prefill(const void* q, long q_stride, const void* k, long
 // =====================================================================================================
 struct DecodeArgs {
     const bf16_t* q; long q_stride; int H, KV; const int* new_len; const int* table; int table_w;
-    const bf16_t* k_pool; const bf16_t* v_pool; int page, rows_cap; float scale, cap; int window;
+    bf16_t* k_pool; bf16_t* v_pool; int page, rows_cap; float scale, cap; int window;
     bf16_t* out; float* ws_o; float* ws_ml; int nsplit;
+    // the step's projections, when the kernel rotates and caches them itself (else null): rows of
+    // [heads | kv heads (keys) | kv heads (values)] x head size, bf16, or float32 in K slices that are added here
+    const void* qkv; int qkv_f32, n_slices; long slice_stride, row_stride;
+    const float* inv_freq; int rot, write_kv;
 };
 
 namespace {
@@ -309,6 +313,7 @@ attn_decode_k(DecodeArgs a) {
     __shared__ float alpha_lds[4][QT];
     __shared__ float m_w[4][QT], l_w[4][QT];
     __shared__ float red[4 * KGW * HD];
+    __shared__ __attribute__((aligned(16))) bf16_t q_lds[QT * HD];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = lane & 15, g = lane >> 4;
     const int kvh = blockIdx.x, seq = blockIdx.y, split = blockIdx.z;
     const int G = a.H / a.KV;
@@ -343,12 +348,70 @@ attn_decode_k(DecodeArgs a) {
         return (((size_t)pg * a.KV + kvh) * a.page + (row & page_mask)) * HD;
     };
 
+    // ---- the group's queries into LDS; in the fused form from the step's projections: K slices added, queries and
+    // the new key rotated (pair (f, f + rot/2), angle p * inv_freq[f], in float32), and the slice that holds position
+    // p writes the key and the value into the cache before anyone in the block reads that row ---------------------
+    if (a.qkv) {
+        const int half = a.rot >> 1, rest = HD - a.rot;
+        auto val = [&](long col) -> float {
+            if (a.qkv_f32) {
+                const float* src = (const float*)a.qkv + (size_t)seq * a.row_stride + col;
+                float t = src[0];
+                for (int sl = 1; sl < a.n_slices; sl++) t += src[(size_t)sl * a.slice_stride];
+                return t;
+            }
+            return bf16_to_f32(((const bf16_t*)a.qkv)[(size_t)seq * a.row_stride + col]);
+        };
+        for (int idx = tid; idx < G * half; idx += DTH) {
+            const int qi = idx / half, f = idx - qi * half;
+            const long col = (long)(kvh * G + qi) * HD;
+            const float ang = (float)p * a.inv_freq[f];
+            const float cs = cosf(ang), sn = sinf(ang);
+            const float x0 = val(col + f), x1 = val(col + f + half);
+            q_lds[qi * HD + f] = f32_to_bf16(x0 * cs - x1 * sn);
+            q_lds[qi * HD + f + half] = f32_to_bf16(x1 * cs + x0 * sn);
+        }
+        for (int idx = tid; idx < G * rest; idx += DTH) {
+            const int qi = idx / rest, d = a.rot + idx - qi * rest;
+            q_lds[qi * HD + d] = f32_to_bf16(val((long)(kvh * G + qi) * HD + d));
+        }
+        if (a.write_kv && p < t_begin + chunk) {                  // t_begin <= p holds here: this slice has position p
+            int row = a.rows_cap > 0 ? p % a.rows_cap : p;
+            const int pg = table[row >> page_shift];
+            const size_t at = (((size_t)pg * a.KV + kvh) * a.page + (row & page_mask)) * HD;
+            bf16_t* kdst = a.k_pool + at;
+            bf16_t* vdst = a.v_pool + at;
+            const long kcol = (long)(a.H + kvh) * HD, vcol = (long)(a.H + a.KV + kvh) * HD;
+            for (int f = tid; f < half; f += DTH) {
+                const float ang = (float)p * a.inv_freq[f];
+                const float cs = cosf(ang), sn = sinf(ang);
+                const float x0 = val(kcol + f), x1 = val(kcol + f + half);
+                kdst[f] = f32_to_bf16(x0 * cs - x1 * sn);
+                kdst[f + half] = f32_to_bf16(x1 * cs + x0 * sn);
+                vdst[f] = f32_to_bf16(val(vcol + f));
+                vdst[f + half] = f32_to_bf16(val(vcol + f + half));
+            }
+            for (int d = a.rot + tid; d < HD; d += DTH) {
+                kdst[d] = f32_to_bf16(val(kcol + d));
+                vdst[d] = f32_to_bf16(val(vcol + d));
+            }
+            __threadfence_block();
+        }
+    } else {
+        for (int idx = tid; idx < G * HD; idx += DTH)
+            q_lds[idx] = a.q[(size_t)seq * a.q_stride + (size_t)kvh * G * HD + idx];
+    }
+    __syncthreads();
     bf16x8 qf[DSTEPS];
 #pragma unroll
     for (int ks = 0; ks < DSTEPS; ks++) {
         const int d0 = dofs(ks, g);
         const bool ok = c < G && d0 < HD;
-        qf[ks] = ld_frag(a.q + (size_t)seq * a.q_stride + (size_t)(kvh * G + (ok ? c : 0)) * HD + (ok ? d0 : 0), ok);
+        Frag f;
+        f.u = *reinterpret_cast<const uint4*>(q_lds + (ok ? c * HD + d0 : 0));
+        const uint32_t keep = (uint32_t) - (int)ok;
+        f.u.x &= keep; f.u.y &= keep; f.u.z &= keep; f.u.w &= keep;
+        qf[ks] = f.v;
     }
     // the lane's part in the weighted sum: chunk ch of the head, keys kgw, kgw + KGW, ... of the wave's 16
     const int ch = lane % NCH, kgw = lane / NCH;
@@ -476,23 +539,51 @@ attn_decode_k(DecodeArgs a) {
     }
 }
 
-__global__ void attn_decode_combine_k(const float* __restrict__ ws_o, const float* __restrict__ ws_ml, int nsplit,
-                                      bf16_t* __restrict__ out) {
+// The slices of one (sequence, head): weights exp(m_s - max m) / sum, computed once by the first wave, then every
+// thread adds its head elements in slice order.  Loads are unconditional (a slice without keys left its sum
+// unwritten: its weight is zero and the value is replaced by zero).
+__global__ void __launch_bounds__(256)
+attn_decode_combine_k(const float* __restrict__ ws_o, const float* __restrict__ ws_ml, int nsplit,
+                      bf16_t* __restrict__ out) {
+    __shared__ float w_lds[128];
     const size_t at = (size_t)blockIdx.x * nsplit;               // blockIdx.x = sequence * heads + head
-    float mx = -INFINITY;
-    for (int s = 0; s < nsplit; s++) mx = fmaxf(mx, ws_ml[(at + s) * 2]);
-    float den = 0.f;
-    for (int s = 0; s < nsplit; s++) {
-        const float m = ws_ml[(at + s) * 2];
-        if (m != -INFINITY) den += __expf(m - mx) * ws_ml[(at + s) * 2 + 1];
+    const int tid = threadIdx.x;
+    if (tid < 64) {
+        const int s0 = tid < nsplit ? tid : nsplit - 1, s1 = tid + 64 < nsplit ? tid + 64 : nsplit - 1;
+        const float2 ml0 = *reinterpret_cast<const float2*>(ws_ml + (at + s0) * 2);
+        const float2 ml1 = *reinterpret_cast<const float2*>(ws_ml + (at + s1) * 2);
+        const float m0 = tid < nsplit ? ml0.x : -INFINITY, m1 = tid + 64 < nsplit ? ml1.x : -INFINITY;
+        float mx = fmaxf(m0, m1);
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+        const float w0 = m0 == -INFINITY ? 0.f : __expf(m0 - mx), w1 = m1 == -INFINITY ? 0.f : __expf(m1 - mx);
+        // the sum in slice order, so that it does not depend on how lanes are paired
+        w_lds[tid] = w0 * ml0.y;
+        w_lds[tid + 64] = w1 * ml1.y;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        float den = 0.f;
+        for (int s = 0; s < nsplit; s++) den += w_lds[s];
+        __builtin_amdgcn_wave_barrier();
+        w_lds[tid] = w0 / den;
+        w_lds[tid + 64] = w1 / den;
     }
-    for (int d = threadIdx.x; d < HD; d += blockDim.x) {
+    __syncthreads();
+    for (int d = tid; d < HD; d += blockDim.x) {
         float num = 0.f;
-        for (int s = 0; s < nsplit; s++) {
-            const float m = ws_ml[(at + s) * 2];
-            if (m != -INFINITY) num += __expf(m - mx) * ws_o[(at + s) * HD + d];
+        for (int s0 = 0; s0 < nsplit; s0 += 8) {
+            float o[8], w[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const int s = s0 + j < nsplit ? s0 + j : nsplit - 1;
+                o[j] = ws_o[(at + s) * HD + d];
+                w[j] = s0 + j < nsplit ? w_lds[s] : 0.f;
+            }
+#pragma unroll
+            for (int j = 0; j < 8; j++) num += w[j] == 0.f ? 0.f : w[j] * o[j];
         }
-        out[(size_t)blockIdx.x * HD + d] = f32_to_bf16(num / den);
+        out[(size_t)blockIdx.x * HD + d] = f32_to_bf16(num);
     }
 }
 
@@ -500,37 +591,61 @@ extern "C" long tp_attn_decode_workspace_floats(int n_seq, int H, int nsplit) {
     return nsplit > 1 ? (long)n_seq * H * nsplit * (HD + 2) : 0;
 }
 
-extern "C" int tp_attn_decode(const void* q, long q_stride, int n_seq, int H, int KV, const int* new_len,
-                              const int* table, int table_w, const void* k_pool, const void* v_pool, int page,
-                              int rows_cap, float scale, float cap, int window, void* out, void* workspace,
-                              int nsplit, void* stream) {
-    TP_REQUIRE(n_seq > 0 && H > 0 && KV > 0, "attention decode: empty shape");
-    TP_REQUIRE(H % KV == 0, "attention: %d query heads are no multiple of %d kv heads", H, KV);
-    const int G = H / KV;
+static int decode_launch(DecodeArgs a, int n_seq, void* workspace, hipStream_t s) {
+    TP_REQUIRE(n_seq > 0 && a.H > 0 && a.KV > 0, "attention decode: empty shape");
+    TP_REQUIRE(a.H % a.KV == 0, "attention: %d query heads are no multiple of %d kv heads", a.H, a.KV);
+    const int G = a.H / a.KV;
     TP_REQUIRE(G <= 16, "attention decode (matrix-core kernel): %d query heads per kv head exceed 16", G);
-    TP_REQUIRE(page >= 16 && (page & (page - 1)) == 0 && table_w > 0, "attention decode (matrix-core kernel): page size %d must be a power of two, at least 16", page);
-    TP_REQUIRE(rows_cap == 0 || window <= rows_cap, "attention decode: a window of %d keys does not fit a ring of %d rows", window, rows_cap);
-    TP_REQUIRE(rows_cap >= 0 && rows_cap % page == 0, "attention decode: ring of %d rows is no multiple of the page size %d", rows_cap, page);
-    TP_REQUIRE(nsplit >= 1 && (nsplit == 1 || workspace), "attention decode: %d slices need a workspace", nsplit);
-    TP_REQUIRE(q_stride % 8 == 0 && (uintptr_t)q % 16 == 0, "attention decode: query rows must be 16-byte aligned");
-    TP_REQUIRE(KV <= 65535 * 1 && n_seq <= 65535 && nsplit <= 65535, "attention decode: grid too large");
-    DecodeArgs a{(const bf16_t*)q, q_stride, H, KV, new_len, table, table_w, (const bf16_t*)k_pool, (const bf16_t*)v_pool,
-                 page, rows_cap, scale, cap, window, (bf16_t*)out, nullptr, nullptr, nsplit};
-    if (nsplit > 1) {
+    TP_REQUIRE(a.page >= 16 && (a.page & (a.page - 1)) == 0 && a.table_w > 0, "attention decode (matrix-core kernel): page size %d must be a power of two, at least 16", a.page);
+    TP_REQUIRE(a.rows_cap == 0 || a.window <= a.rows_cap, "attention decode: a window of %d keys does not fit a ring of %d rows", a.window, a.rows_cap);
+    TP_REQUIRE(a.rows_cap >= 0 && a.rows_cap % a.page == 0, "attention decode: ring of %d rows is no multiple of the page size %d", a.rows_cap, a.page);
+    TP_REQUIRE(a.nsplit >= 1 && a.nsplit <= 128 && (a.nsplit == 1 || workspace), "attention decode: %d slices (at most 128) need a workspace", a.nsplit);
+    TP_REQUIRE(a.KV <= 65535 && n_seq <= 65535, "attention decode: grid too large");
+    if (a.nsplit > 1) {
         a.ws_o = (float*)workspace;
-        a.ws_ml = a.ws_o + (size_t)n_seq * H * nsplit * HD;
+        a.ws_ml = a.ws_o + (size_t)n_seq * a.H * a.nsplit * HD;
     }
-    dim3 grid(KV, n_seq, nsplit);
-    hipStream_t s = (hipStream_t)stream;
+    dim3 grid(a.KV, n_seq, a.nsplit);
     if (G <= 1) attn_decode_k<1><<<grid, DTH, 0, s>>>(a);
     else if (G <= 2) attn_decode_k<2><<<grid, DTH, 0, s>>>(a);
     else if (G <= 4) attn_decode_k<4><<<grid, DTH, 0, s>>>(a);
     else if (G <= 8) attn_decode_k<8><<<grid, DTH, 0, s>>>(a);
     else attn_decode_k<16><<<grid, DTH, 0, s>>>(a);
     if (int rc = tp_check_launch("attention decode")) return rc;
-    if (nsplit > 1) {
-        attn_decode_combine_k<<<n_seq * H, HD < 64 ? 64 : HD, 0, s>>>(a.ws_o, a.ws_ml, nsplit, (bf16_t*)out);
+    if (a.nsplit > 1) {
+        attn_decode_combine_k<<<n_seq * a.H, HD < 64 ? 64 : HD, 0, s>>>(a.ws_o, a.ws_ml, a.nsplit, a.out);
         return tp_check_launch("attention decode (combine)");
     }
     return 0;
+}
+
+extern "C" int tp_attn_decode(const void* q, long q_stride, int n_seq, int H, int KV, const int* new_len,
+                              const int* table, int table_w, const void* k_pool, const void* v_pool, int page,
+                              int rows_cap, float scale, float cap, int window, void* out, void* workspace,
+                              int nsplit, void* stream) {
+    TP_REQUIRE(q_stride % 8 == 0 && (uintptr_t)q % 16 == 0, "attention decode: query rows must be 16-byte aligned");
+    DecodeArgs a{(const bf16_t*)q, q_stride, H, KV, new_len, table, table_w, (bf16_t*)k_pool, (bf16_t*)v_pool,
+                 page, rows_cap, scale, cap, window, (bf16_t*)out, nullptr, nullptr, nsplit,
+                 nullptr, 0, 1, 0, 0, nullptr, 0, 0};
+    return decode_launch(a, n_seq, workspace, (hipStream_t)stream);
+}
+
+// One launch for a decode step's rotation, cache write and attention: `qkv` holds each sequence's projections
+// [heads | kv heads (keys) | kv heads (values)] x head size (queries only when write_kv is 0) as bf16 rows, or as
+// float32 rows in n_slices K slices `slice_stride` elements apart.  Sequence i's new token has position new_len[i] - 1.
+extern "C" int tp_attn_decode_fused(const void* qkv, int qkv_dtype, int n_slices, long slice_stride, long row_stride,
+                                    const float* inv_freq, int rot, int write_kv,
+                                    int n_seq, int H, int KV, const int* new_len, const int* table, int table_w,
+                                    void* k_pool, void* v_pool, int page, int rows_cap, float scale, float cap,
+                                    int window, void* out, void* workspace, int nsplit, void* stream) {
+    TP_REQUIRE(qkv, "attention decode (fused): no projections");
+    TP_REQUIRE(qkv_dtype == TP_BF16 || qkv_dtype == TP_F32, "attention decode (fused): projections of dtype %d", qkv_dtype);
+    TP_REQUIRE(n_slices >= 1 && (n_slices == 1 || qkv_dtype == TP_F32), "attention decode (fused): %d slices must be float32", n_slices);
+    TP_REQUIRE(rot >= 0 && rot <= HD && rot % 2 == 0, "attention decode (fused): rotary_dim %d must be even and at most head_dim %d", rot, HD);
+    TP_REQUIRE(rot == 0 || inv_freq, "attention decode (fused): a rotation needs its frequency table");
+    TP_REQUIRE(row_stride >= (long)(H + (write_kv ? 2 * KV : 0)) * HD, "attention decode (fused): rows of %ld elements are too short", row_stride);
+    DecodeArgs a{nullptr, 0, H, KV, new_len, table, table_w, (bf16_t*)k_pool, (bf16_t*)v_pool,
+                 page, rows_cap, scale, cap, window, (bf16_t*)out, nullptr, nullptr, nsplit,
+                 qkv, qkv_dtype == TP_F32 ? 1 : 0, n_slices, slice_stride, row_stride, inv_freq, rot, write_kv};
+    return decode_launch(a, n_seq, workspace, (hipStream_t)stream);
 }

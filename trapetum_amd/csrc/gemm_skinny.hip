@@ -72,7 +72,7 @@ gemm_skinny_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* 
     auto load = [&](int kw, bf16x8 (&a)[U][NT], bf16x8 (&b)[U][MT]) {
 #pragma unroll
         for (int u = 0; u < U; u++) {
-            const int k = kw + u * 128 + g * 8;
+            const int k = kw + (u >> 1) * 256 + (u & 1) * 32 + g * 8;
             const bool ok = k < kend;
             const int kc = ok ? k : klast;
 #pragma unroll
@@ -101,7 +101,7 @@ gemm_skinny_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* 
                     acc[s][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][s], b[u][t], acc[s][t], 0, 0, 0);
     };
     bf16x8 a0[U][NT], b0[U][MT], a1[U][NT], b1[U][MT];
-    int kw = kbeg + wave * 32;
+    int kw = kbeg + wave * 64;
     if (kw < kend) {
         load(kw, a0, b0);
         while (true) {

@@ -34,6 +34,7 @@ _ATTN_SIGS = {
     "tp_attn_prefill_workspace_elems": [_I, _I, _I],
     "tp_attn_decode": [_P, _L, _I, _I, _I, _P, _P, _I, _P, _P, _I, _I, _F, _F, _I, _P, _P, _I, _P],
     "tp_attn_decode_workspace_floats": [_I, _I, _I],
+    "tp_attn_decode_fused": [_P, _I, _I, _L, _L, _P, _I, _I, _I, _I, _I, _P, _P, _I, _P, _P, _I, _I, _F, _F, _I, _P, _P, _I, _P],
 }
 
 EPI_NONE, EPI_SOFTCAP, EPI_GATED = 0, 1, 2
@@ -295,25 +296,41 @@ class HipOps:
                    int(window), out.data_ptr(), self._stream())
         return out
 
+    @staticmethod
+    def decode_splits(n, KV, hd, keys):
+        """Slices of the keys per (sequence, kv head) in a decode step.  A block streams about 85 GB/s and the chip
+        holds about 512 blocks at once; several slices cost a second launch that adds them (about 5 us)."""
+        best, best_t = 1, None
+        for ns in range(1, min(128, -(-keys // 64)) + 1):
+            per_block = -(-keys // ns) * hd * 4 / 85e3                   # us: keys and values, 2 bytes each
+            t = per_block * -(-(n * KV * ns) // 512) + (5.0 if ns > 1 else 0.0)
+            if best_t is None or t < best_t - 1e-9:
+                best, best_t = ns, t
+        return best
+
+    def _decode_pools(self, what, dtype, n, KV, hd, new_len, table, k_pool, v_pool):
+        if new_len.numel() != n or new_len.dtype != torch.int32:
+            raise KernelError(f"{what}: one int32 length per sequence")
+        if k_pool.dtype != dtype or k_pool.dim() != 4 or tuple(k_pool.shape[1:]) != (KV, k_pool.shape[2], hd) \
+                or v_pool.shape != k_pool.shape or not k_pool.is_contiguous() or not v_pool.is_contiguous():
+            raise KernelError(f"{what}: cache pools must be contiguous [pages, kv_heads, page, head_dim] of {dtype}")
+        if table.dtype != torch.int32 or table.dim() != 2 or table.shape[0] != n or not table.is_contiguous():
+            raise KernelError(f"{what}: the page table must be contiguous int32 [sequences, pages]")
+
     def attention_decode(self, q, H, KV, hd, new_len, table, k_pool, v_pool, rows_cap, scale, softcap, window,
-                         out_dtype, max_keys=None):
+                         out_dtype, max_keys=None, splits=None):
         self._dev(q, new_len, table, k_pool, v_pool)
         n = q.shape[0]
         qs = self._rows(q, "attention q")
-        if q.shape[1] != H * hd or new_len.numel() != n or new_len.dtype != torch.int32:
-            raise KernelError("attention_decode: q must be [sequences, heads * head_dim] with one int32 length each")
-        if k_pool.dtype != q.dtype or k_pool.dim() != 4 or tuple(k_pool.shape[1:]) != (KV, k_pool.shape[2], hd) \
-                or v_pool.shape != k_pool.shape or not k_pool.is_contiguous() or not v_pool.is_contiguous():
-            raise KernelError("attention_decode: cache pools must be contiguous [pages, kv_heads, page, head_dim] of q's dtype")
-        if table.dtype != torch.int32 or table.dim() != 2 or table.shape[0] != n or not table.is_contiguous():
-            raise KernelError("attention_decode: the page table must be contiguous int32 [sequences, pages]")
+        if q.shape[1] != H * hd:
+            raise KernelError("attention_decode: q must be [sequences, heads * head_dim]")
+        self._decode_pools("attention_decode", q.dtype, n, KV, hd, new_len, table, k_pool, v_pool)
         out = torch.empty((n, H * hd), dtype=out_dtype, device=self.device)
         page = k_pool.shape[2]
         if self._fast_attention(q.dtype, H, KV, hd) and page >= 16 and page & (page - 1) == 0:
             lib = self.attn_lib(hd)
             keys = int(max_keys) if max_keys else k_pool.shape[0] * k_pool.shape[2]
-            # enough blocks to fill the chip, each with at least one round of 64 keys
-            nsplit = max(1, min(-(-768 // (n * KV)), -(-keys // 64), 128))
+            nsplit = int(splits) if splits else self.decode_splits(n, KV, hd, keys)
             floats = lib.tp_attn_decode_workspace_floats(n, H, nsplit)
             ws = torch.empty(floats, dtype=torch.float32, device=self.device) if floats else None
             self._call(lib, "tp_attn_decode", q.data_ptr(), qs, n, H, KV, new_len.data_ptr(), table.data_ptr(),
@@ -324,6 +341,49 @@ class HipOps:
         self._call(self.lib, "tp_attn_simple_decode", q.data_ptr(), qs, _code(q.dtype), n, H, KV, hd, new_len.data_ptr(),
                    table.data_ptr(), table.shape[1], k_pool.data_ptr(), v_pool.data_ptr(), k_pool.shape[2], rows_cap,
                    float(scale), float(softcap), int(window), out.data_ptr(), self._stream())
+        return out
+
+    def fuses_decode_step(self, dtype, H, KV, hd, k_pool):
+        """Whether `attention_decode_step` exists for this geometry: the caller then skips `rope_kv_write`."""
+        page = k_pool.shape[2]
+        return self._fast_attention(dtype, H, KV, hd) and page >= 16 and page & (page - 1) == 0
+
+    def attention_decode_step(self, qkv, H, KV, hd, inv_freq, rotary_dim, new_len, table, k_pool, v_pool, rows_cap,
+                              scale, softcap, window, out_dtype, max_keys=None, write_kv=True, splits=None):
+        """A decode step's rotation, cache write and attention in one launch.  qkv: each sequence's projections
+        [queries | keys | values] (queries only when write_kv is false), a bf16 tensor or what
+        `linear(..., defer=True)` returned; sequence i's token has position new_len[i] - 1."""
+        split = isinstance(qkv, SplitRows)
+        rows = qkv.slices if split else qkv
+        self._dev(rows, inv_freq, new_len, table, k_pool, v_pool)
+        n, width = rows.shape[-2], rows.shape[-1]
+        if width != (H + (2 * KV if write_kv else 0)) * hd:
+            raise KernelError(f"attention_decode_step: rows of {width} columns, {H} heads and {KV} kv heads of {hd} need "
+                              f"{(H + (2 * KV if write_kv else 0)) * hd}")
+        if out_dtype != torch.bfloat16 or not self.fuses_decode_step(out_dtype, H, KV, hd, k_pool):
+            raise KernelError("attention_decode_step: no fused kernel for this geometry (see fuses_decode_step)")
+        if split:
+            if rows.dtype != torch.float32 or not rows.is_contiguous():
+                raise KernelError("attention_decode_step: K slices must be contiguous float32")
+            n_slices, slice_stride, row_stride = rows.shape[0], rows.shape[1] * rows.shape[2], rows.shape[2]
+        else:
+            if rows.dim() != 2 or rows.dtype not in (torch.bfloat16, torch.float32):
+                raise KernelError("attention_decode_step: projections must be 2-D, bfloat16 or float32")
+            n_slices, slice_stride, row_stride = 1, 0, self._rows(rows, "attention_decode_step qkv")
+        if rotary_dim and (inv_freq is None or inv_freq.dtype != torch.float32 or inv_freq.numel() != rotary_dim // 2):
+            raise KernelError(f"attention_decode_step: a rotation over {rotary_dim} needs float32 inv_freq [{rotary_dim // 2}]")
+        self._decode_pools("attention_decode_step", torch.bfloat16, n, KV, hd, new_len, table, k_pool, v_pool)
+        lib = self.attn_lib(hd)
+        keys = int(max_keys) if max_keys else k_pool.shape[0] * k_pool.shape[2]
+        nsplit = int(splits) if splits else self.decode_splits(n, KV, hd, keys)
+        floats = lib.tp_attn_decode_workspace_floats(n, H, nsplit)
+        ws = torch.empty(floats, dtype=torch.float32, device=self.device) if floats else None
+        out = torch.empty((n, H * hd), dtype=out_dtype, device=self.device)
+        self._call(lib, "tp_attn_decode_fused", rows.data_ptr(), _code(rows.dtype), n_slices, slice_stride, row_stride,
+                   inv_freq.data_ptr() if rotary_dim else None, int(rotary_dim), 1 if write_kv else 0,
+                   n, H, KV, new_len.data_ptr(), table.data_ptr(), table.shape[1], k_pool.data_ptr(), v_pool.data_ptr(),
+                   k_pool.shape[2], rows_cap, float(scale), float(softcap), int(window), out.data_ptr(),
+                   ws.data_ptr() if ws is not None else None, nsplit, self._stream())
         return out
 
     # ---- token choice -------------------------------------------------------------------------------------

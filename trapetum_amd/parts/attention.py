@@ -55,13 +55,20 @@ class Attention(Mixer):
         H, KV, hd = self.num_heads, self.num_kv_heads, self.head_dim
         Q, KVD = H * hd, KV * hd
         owns_cache = ctx.cache_owner == ctx.entry
+        table = ctx.page_table(site.group_index)
+        rows_cap = site.rows_cap or 0
+        if ctx.mode == "decode" and ops.fuses_decode_step(ctx.dtype, H, KV, hd, site.k):
+            # one launch rotates, writes the cache and attends; the projections may stay in K slices until then
+            qkv = ops.linear(x, self.w_qkv if owns_cache else self.w_qkv[:Q], ctx.dtype, defer=True)
+            out = ops.attention_decode_step(qkv, H, KV, hd, self.inv_freq, self.position.rotary_dim, ctx.new_len,
+                                            table, site.k, site.v, rows_cap, self.query_scale, self.softcap,
+                                            self.window, ctx.dtype, max_keys=ctx.max_keys(site), write_kv=owns_cache)
+            return ops.linear(out, self.w_o, ctx.dtype, defer=True)
         if owns_cache:
             qkv = ops.linear(x, self.w_qkv, ctx.dtype)
             q, k, v = qkv[:, :Q], qkv[:, Q:Q + KVD], qkv[:, Q + KVD:]
         else:
             q, k, v = ops.linear(x, self.w_qkv[:Q], ctx.dtype), None, None
-        table = ctx.page_table(site.group_index)
-        rows_cap = site.rows_cap or 0
         ops.rope_kv_write(q, k, v, H, KV, hd, self.inv_freq, self.position.rotary_dim,
                           ctx.row_seq, ctx.row_pos, ctx.new_len, table, site.k, site.v, rows_cap)
         if ctx.mode == "prefill":
