@@ -348,6 +348,38 @@ attn_decode_k(DecodeArgs a) {
         return (((size_t)pg * a.KV + kvh) * a.page + (row & page_mask)) * HD;
     };
 
+    // the lane's part in the weighted sum: chunk ch of the head, keys kgw, kgw + KGW, ... of the wave's 16
+    const int ch = lane % NCH, kgw = lane / NCH;
+    const bool pv_lane = kgw < KGW;
+    // ---- loads of a round: the key row of lane c for the scores, value chunks for the sum.  Unconditional loads of
+    // rows that exist: a hidden or surplus key gets probability 0 (or is skipped) in the sum ---------------------
+    auto load_round = [&](int tb, bf16x8 (&kf)[DSTEPS], Frag (&vf)[VPT]) {
+        const size_t tile = tile_offset(__builtin_amdgcn_readfirstlane(tb));
+        int tk = tb + c;
+        tk = tk < lo ? lo : (tk > p ? p : tk);
+        const bf16_t* kp = a.k_pool + tile + (size_t)(tk - tb) * HD;
+#pragma unroll
+        for (int ks = 0; ks < DSTEPS; ks++) {
+            const int d0 = dofs(ks, g);
+            kf[ks] = ld_frag(kp + (d0 < HD ? d0 : 0), d0 < HD);
+        }
+#pragma unroll
+        for (int j = 0; j < VPT; j++) {
+            int kk = kgw + j * KGW;
+            kk = kk > 15 ? 15 : kk;
+            int tv = tb + kk;
+            tv = tv < lo ? lo : (tv > p ? p : tv);
+            vf[j].u = *reinterpret_cast<const uint4*>(a.v_pool + tile + (size_t)(tv - tb) * HD + ch * 8);
+        }
+    };
+    // The wave's first round is fetched while the queries are prepared, unless its tile holds the row that this
+    // block is about to write.
+    bf16x8 kf[DSTEPS];
+    Frag vf[VPT];
+    const int tb0 = t_begin + wave * 16;
+    const bool late = a.qkv && a.write_kv && tb0 <= p && p < tb0 + 16;
+    if (tb0 < t_end && !late) load_round(tb0, kf, vf);
+
     // ---- the group's queries into LDS; in the fused form from the step's projections: K slices added, queries and
     // the new key rotated (pair (f, f + rot/2), angle p * inv_freq[f], in float32), and the slice that holds position
     // p writes the key and the value into the cache before anyone in the block reads that row ---------------------
@@ -413,9 +445,6 @@ attn_decode_k(DecodeArgs a) {
         f.u.x &= keep; f.u.y &= keep; f.u.z &= keep; f.u.w &= keep;
         qf[ks] = f.v;
     }
-    // the lane's part in the weighted sum: chunk ch of the head, keys kgw, kgw + KGW, ... of the wave's 16
-    const int ch = lane % NCH, kgw = lane / NCH;
-    const bool pv_lane = kgw < KGW;
     float acc[QT][8];
 #pragma unroll
     for (int qi = 0; qi < QT; qi++)
@@ -424,27 +453,8 @@ attn_decode_k(DecodeArgs a) {
     float m_run = -INFINITY, l_run = 0.f;            // of query head c, over this wave's keys so far
     const float soc = a.cap > 0.f ? a.scale / a.cap : 0.f;
 
-    for (int tb = t_begin + wave * 16; tb < t_end; tb += ROUND) {
-        // ---- loads of the round: the key row of lane c for the scores, value chunks for the sum ------------------
-        const size_t tile = tile_offset(__builtin_amdgcn_readfirstlane(tb));
-        int tk = tb + c;
-        tk = tk < lo ? lo : (tk > p ? p : tk);                   // a row that exists; masked below
-        const bf16_t* kp = a.k_pool + tile + (size_t)(tk - tb) * HD;
-        bf16x8 kf[DSTEPS];
-#pragma unroll
-        for (int ks = 0; ks < DSTEPS; ks++) {
-            const int d0 = dofs(ks, g);
-            kf[ks] = ld_frag(kp + (d0 < HD ? d0 : 0), d0 < HD);
-        }
-        Frag vf[VPT];
-#pragma unroll
-        for (int j = 0; j < VPT; j++) {              // unconditional loads of rows that exist: a hidden or surplus
-            int kk = kgw + j * KGW;                  // key gets probability 0 (or is skipped) in the sum below
-            kk = kk > 15 ? 15 : kk;
-            int tv = tb + kk;
-            tv = tv < lo ? lo : (tv > p ? p : tv);
-            vf[j].u = *reinterpret_cast<const uint4*>(a.v_pool + tile + (size_t)(tv - tb) * HD + ch * 8);
-        }
+    for (int tb = tb0; tb < t_end; tb += ROUND) {
+        if (tb != tb0 || late) load_round(tb, kf, vf);
         // ---- scores of 16 keys for the group's query heads: lane (c, g) gets keys g*4 .. g*4+3 of head c ----------
         f32x4 s = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -506,8 +516,9 @@ attn_decode_k(DecodeArgs a) {
     }
     // ---- the four waves' results: rescale to a common maximum, add in wave and key-group order, write -------------
     if (c < QT && g == 0) { m_w[wave][c] = m_run; l_w[wave][c] = l_run; }
+#pragma unroll
     for (int qi = 0; qi < QT; qi++) {
-        if (qi >= G) break;
+        if (qi >= G) continue;                       // G is the same for the whole block; unrolled, so that acc stays in registers
         if (pv_lane) {
 #pragma unroll
             for (int e = 0; e < 8; e++) red[(wave * KGW + kgw) * HD + ch * 8 + e] = acc[qi][e];

@@ -298,15 +298,19 @@ class HipOps:
 
     @staticmethod
     def decode_splits(n, KV, hd, keys):
-        """Slices of the keys per (sequence, kv head) in a decode step.  A block streams about 85 GB/s and the chip
-        holds about 512 blocks at once; several slices cost a second launch that adds them (about 5 us)."""
-        best, best_t = 1, None
+        """Slices of the keys per (sequence, kv head) in a decode step, from a fit to measurements on MI355X: a block
+        streams about 32 GB/s, 768 blocks run at once, the chip delivers about 5.5 TB/s (and half of that time is
+        felt even when blocks are few), and several slices cost a second launch that adds them.  The fewest slices
+        within 3 % of the best estimate."""
+        per_pair = keys * hd * 4                                         # bytes of keys and values, 2 bytes each
+        floor = n * KV * per_pair / 5.5e6
+        est = []
         for ns in range(1, min(128, -(-keys // 64)) + 1):
-            per_block = -(-keys // ns) * hd * 4 / 85e3                   # us: keys and values, 2 bytes each
-            t = per_block * -(-(n * KV * ns) // 512) + (5.0 if ns > 1 else 0.0)
-            if best_t is None or t < best_t - 1e-9:
-                best, best_t = ns, t
-        return best
+            rounds = -(-(n * KV * ns) // 768)
+            t = max(per_pair / ns / 32e3 * rounds + 0.5 * floor, floor)
+            est.append(t + (2.5 + 0.05 * ns if ns > 1 else 0.0))
+        best = min(est)
+        return next(i + 1 for i, t in enumerate(est) if t <= best * 1.03 + 1e-9)
 
     def _decode_pools(self, what, dtype, n, KV, hd, new_len, table, k_pool, v_pool):
         if new_len.numel() != n or new_len.dtype != torch.int32:
