@@ -52,9 +52,9 @@ __device__ __forceinline__ bf16_t bf16_bits(float f) {
 
 // =====================================================================================================
 // prefill: every sequence of the step starts at position 0; keys and values are the step's own rows.
-// Block = 4 waves = 64 queries of one (sequence, head); each wave owns 16 queries.  Key tiles of 32 go
-// through LDS: K as stored (row = key), V transposed (row = head element) with the keys of a tile permuted
-// so that a lane's 8 probabilities meet the 8 values of the same keys in one 16-byte LDS read.
+// Block = 64 queries of one (sequence, head); a wave owns 16 queries.  Key tiles of 32 go through LDS: K as
+// stored (row = key), V transposed (row = head element) with the keys of a tile permuted so that a lane's 8
+// probabilities meet the 8 values of the same keys in one 16-byte LDS read.
 // =====================================================================================================
 struct PrefillArgs {
     const bf16_t* q; long q_stride; const bf16_t* k; long k_stride; const bf16_t* v; long v_stride;
@@ -101,11 +101,29 @@ v_transpose_k(const bf16_t* __restrict__ v, long v_stride, int KV, const int* __
     }
 }
 
-__global__ void __launch_bounds__(256)
+// Block = 8 waves in two groups of four, 64 queries of one (sequence, head): wave w of either group owns queries
+// w*16 .. w*16+15.  Per round the block stages two key tiles (64 keys); group 0 takes the first, group 1 the
+// second, each with its own running softmax, so the chain of dependent rounds is half as long as the keys; at
+// the end group 1 hands (max, sum, unnormalised output) to group 0 through LDS.
+namespace {
+constexpr int PTH = 512;                                         // threads of a prefill block
+constexpr int PGROUPS = 2;
+constexpr int PKEYS = PGROUPS * BKV;                             // keys staged per round
+constexpr int KS_ELEMS = BKV * KLD, VT_ELEMS = HD * VLD;         // one tile's K and V^T in LDS
+constexpr int MERGE_LANE = HD / 4 + 4;                           // group 1's state per lane: its output tiles, max, sum (16-byte rows)
+constexpr int MERGE_FLOATS = 4 * 64 * MERGE_LANE;
+constexpr size_t PREFILL_LDS_TILES = (size_t)PGROUPS * (KS_ELEMS + VT_ELEMS) * sizeof(bf16_t);
+constexpr size_t PREFILL_LDS = PREFILL_LDS_TILES > MERGE_FLOATS * sizeof(float) ? PREFILL_LDS_TILES : MERGE_FLOATS * sizeof(float);
+}
+
+__global__ void __launch_bounds__(PTH)
 attn_prefill_k(PrefillArgs a) {
-    __shared__ __attribute__((aligned(16))) bf16_t Ks[BKV * KLD];
-    __shared__ __attribute__((aligned(16))) bf16_t Vt[HD * VLD];
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = lane & 15, g = lane >> 4;
+    extern __shared__ __attribute__((aligned(16))) unsigned char prefill_lds[];
+    bf16_t* Ks_all = reinterpret_cast<bf16_t*>(prefill_lds);                       // [group][BKV][KLD]
+    bf16_t* Vt_all = Ks_all + PGROUPS * KS_ELEMS;                                  // [group][HD][VLD]
+    const int tid = threadIdx.x, grp = tid >> 8, wave = (tid >> 6) & 3, lane = tid & 63, c = lane & 15, g = lane >> 4;
+    const bf16_t* Ks = Ks_all + grp * KS_ELEMS;
+    const bf16_t* Vt = Vt_all + grp * VT_ELEMS;
     // late query tiles see the most keys: they are given the low block ids, which start first
     const int seq = blockIdx.z, h = blockIdx.y, q0 = (gridDim.x - 1 - blockIdx.x) * 64;
     const int row0 = a.cu_rows[seq], T = a.cu_rows[seq + 1] - row0;
@@ -121,7 +139,10 @@ attn_prefill_k(PrefillArgs a) {
         qf[ks] = ld_frag(a.q + (size_t)(row0 + (q_ok ? qpos : 0)) * a.q_stride + (size_t)h * HD + d0, q_ok && d0 < HD);
     }
     if (HDP > HD)                                   // the padding columns of K stay zero for the whole kernel
-        for (int i = tid; i < BKV * (HDP - HD); i += 256) Ks[(i / (HDP - HD)) * KLD + HD + i % (HDP - HD)] = 0;
+        for (int i = tid; i < PKEYS * (HDP - HD); i += PTH) {
+            const int key = i / (HDP - HD);
+            Ks_all[(key / BKV) * KS_ELEMS + (key % BKV) * KLD + HD + i % (HDP - HD)] = 0;
+        }
 
     f32x4 o[HD / 16];
 #pragma unroll
@@ -132,49 +153,54 @@ attn_prefill_k(PrefillArgs a) {
     int k_lo = a.window > 0 ? max(0, q0 - a.window + 1) : 0;
     k_lo &= ~(BKV - 1);
     const int k_hi = min(T, q0 + 64);
-    // a tile's rows travel global memory -> registers (one tile ahead, while the tile before is being used) -> LDS;
-    // K as stored, V from its transposed copy: HD rows of 32 slots (64 bytes) each
-    constexpr int KTASKS = (BKV * NCH + 255) / 256;                 // (key, 16-byte chunk) per thread
-    constexpr int VTASKS = (HD * 4 + 255) / 256;                    // (head element, 16-byte chunk of its 32 slots)
+    // a round's rows travel global memory -> registers (one round ahead, while the round before is being used) ->
+    // LDS; K as stored, V from its transposed copy: HD rows of 64 slots (128 bytes) per round
+    constexpr int KTASKS = (PKEYS * NCH + PTH - 1) / PTH;           // (key, 16-byte chunk) per thread
+    constexpr int VTASKS = (HD * 8 + PTH - 1) / PTH;                // (head element, 16-byte chunk of its 64 slots)
     Frag fk[KTASKS], fv[VTASKS];
     const int vbase = vt_base_of(a.cu_rows, seq);
     auto fetch = [&](int kt) {
 #pragma unroll
         for (int t = 0; t < KTASKS; t++) {
-            const int i = tid + t * 256;
+            const int i = tid + t * PTH;
             const int key = i / NCH, ch = i % NCH, tk = kt + key;
             fk[t].u = make_uint4(0, 0, 0, 0);
-            if (i < BKV * NCH && tk < T)
+            if (i < PKEYS * NCH && tk < T)
                 fk[t].u = *reinterpret_cast<const uint4*>(a.k + (size_t)(row0 + tk) * a.k_stride + (size_t)kvh * HD + ch * 8);
         }
 #pragma unroll
         for (int t = 0; t < VTASKS; t++) {
-            const int i = tid + t * 256;
-            const int d = i >> 2, part = i & 3;
+            const int i = tid + t * PTH;
+            const int d = i >> 3, part = i & 7;
             fv[t].u = make_uint4(0, 0, 0, 0);
-            if (i < HD * 4)
+            if (i < HD * 8 && kt + (part >> 2) * BKV < k_hi)         // a tile past the block's last key is never used
                 fv[t].u = *reinterpret_cast<const uint4*>(a.vt + ((size_t)kvh * HD + d) * a.vt_rows + vbase + kt + part * 8);
         }
     };
     auto stage = [&]() {
 #pragma unroll
         for (int t = 0; t < KTASKS; t++) {
-            const int i = tid + t * 256;
-            if (i < BKV * NCH) *reinterpret_cast<uint4*>(Ks + (i / NCH) * KLD + (i % NCH) * 8) = fk[t].u;
+            const int i = tid + t * PTH;
+            const int key = i / NCH;
+            if (i < PKEYS * NCH)
+                *reinterpret_cast<uint4*>(Ks_all + (key / BKV) * KS_ELEMS + (key % BKV) * KLD + (i % NCH) * 8) = fk[t].u;
         }
 #pragma unroll
         for (int t = 0; t < VTASKS; t++) {
-            const int i = tid + t * 256;
-            if (i < HD * 4) *reinterpret_cast<uint4*>(Vt + (i >> 2) * VLD + (i & 3) * 8) = fv[t].u;
+            const int i = tid + t * PTH;
+            const int d = i >> 3, part = i & 7;                      // slots part*8 .. +7 of the round: tile part / 4
+            if (i < HD * 8)
+                *reinterpret_cast<uint4*>(Vt_all + (part >> 2) * VT_ELEMS + d * VLD + (part & 3) * 8) = fv[t].u;
         }
     };
     fetch(k_lo);
-    for (int kt = k_lo; kt < k_hi; kt += BKV) {
-        __syncthreads();                             // the tile before has been used by every wave
+    for (int kr = k_lo; kr < k_hi; kr += PKEYS) {
+        __syncthreads();                             // the round before has been used by every wave
         stage();
         __syncthreads();
-        if (kt + BKV < k_hi) fetch(kt + BKV);
-        const bool visible = qw0 < T && kt <= qw0 + 15 && !(a.window > 0 && kt + BKV - 1 < qw0 - a.window + 1);
+        if (kr + PKEYS < k_hi) fetch(kr + PKEYS);
+        const int kt = kr + grp * BKV;               // this group's tile
+        const bool visible = kt < k_hi && qw0 < T && kt <= qw0 + 15 && !(a.window > 0 && kt + BKV - 1 < qw0 - a.window + 1);
         if (!visible) continue;                      // wave-uniform: every key of the tile is hidden from the wave's queries
 
         f32x4 s[2];
@@ -236,14 +262,28 @@ attn_prefill_k(PrefillArgs a) {
             o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf.v, o[dt], 0, 0, 0);
         }
     }
-    if (!q_ok) return;
-    const float inv = 1.f / l_i;
+    // ---- group 1's state joins group 0's: both rescaled to the common maximum, group 0 first ---------------------
+    __syncthreads();                                 // the tiles in LDS are done with
+    float* merge = reinterpret_cast<float*>(prefill_lds) + (size_t)(wave * 64 + lane) * MERGE_LANE;
+    if (grp == 1) {
+#pragma unroll
+        for (int dt = 0; dt < HD / 16; dt++) *reinterpret_cast<f32x4*>(merge + dt * 4) = o[dt];
+        merge[HD / 4] = m_i;
+        merge[HD / 4 + 1] = l_i;
+    }
+    __syncthreads();
+    if (grp == 1 || !q_ok) return;
+    const float m1 = merge[HD / 4], l1 = merge[HD / 4 + 1];
+    const float m = fmaxf(m_i, m1);
+    const float a0 = m_i == -INFINITY ? 0.f : __expf(m_i - m), a1 = m1 == -INFINITY ? 0.f : __expf(m1 - m);
+    const float inv = 1.f / (l_i * a0 + l1 * a1);
     bf16_t* orow = a.out + ((size_t)(row0 + qpos) * a.H + h) * HD;
 #pragma unroll
     for (int dt = 0; dt < HD / 16; dt++) {
+        const f32x4 o1 = *reinterpret_cast<const f32x4*>(merge + dt * 4);
         ushort4 pk;
-        pk.x = bf16_bits(o[dt][0] * inv); pk.y = bf16_bits(o[dt][1] * inv);
-        pk.z = bf16_bits(o[dt][2] * inv); pk.w = bf16_bits(o[dt][3] * inv);
+        pk.x = bf16_bits((o[dt][0] * a0 + o1[0] * a1) * inv); pk.y = bf16_bits((o[dt][1] * a0 + o1[1] * a1) * inv);
+        pk.z = bf16_bits((o[dt][2] * a0 + o1[2] * a1) * inv); pk.w = bf16_bits((o[dt][3] * a0 + o1[3] * a1) * inv);
         *reinterpret_cast<ushort4*>(orow + dt * 16 + g * 4) = pk;
     }
 }
@@ -269,8 +309,14 @@ extern "C" int tp_attn_prefill(const void* q, long q_stride, const void* k, long
     if (int rc = tp_check_launch("attention prefill (transpose of V)")) return rc;
     PrefillArgs a{(const bf16_t*)q, q_stride, (const bf16_t*)k, k_stride, (const bf16_t*)v, v_stride, H, KV, cu_rows,
                   scale, cap, window, (bf16_t*)out, (const bf16_t*)workspace, vt_rows};
+    static bool configured = false;                                   // more LDS than a kernel gets without asking
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute((const void*)attn_prefill_k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)PREFILL_LDS);
+        if (e != hipSuccess) return tp_fail("attention prefill: cannot reserve %zu bytes of LDS: %s", (size_t)PREFILL_LDS, hipGetErrorString(e));
+        configured = true;
+    }
     dim3 grid(tp_cdiv(max_count, 64), H, n_seq);
-    attn_prefill_k<<<grid, 256, 0, (hipStream_t)stream>>>(a);
+    attn_prefill_k<<<grid, PTH, PREFILL_LDS, (hipStream_t)stream>>>(a);
     return tp_check_launch("attention prefill");
 }
 
