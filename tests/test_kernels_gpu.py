@@ -177,7 +177,7 @@ def build_cache_case(dt, H, KV, hd, lens, page, rows_cap, n_pages, seed):
 @pytest.mark.parametrize("dt", ["f32", "bf16"])
 @pytest.mark.parametrize("H,KV,hd,lens,page,rows_cap", [
     (4, 2, 16, (5, 11, 17), 16, 0), (6, 1, 32, (1, 9, 23, 40), 16, 16), (3, 3, 48, (70, 3), 64, 64),
-    (8, 4, 256, (130,), 64, 0), (2, 2, 80, (33, 50), 16, 32)])
+    (8, 4, 256, (130,), 64, 0), (2, 2, 80, (33, 50), 16, 32), (4, 2, 64, (200, 90), 16, 0), (5, 1, 32, (300,), 16, 64)])
 def test_rope_kv_write(ops, dt, H, KV, hd, lens, page, rows_cap):
     c = build_cache_case(DT[dt], H, KV, hd, lens, page, rows_cap, 24, 20)
     pools_ref = [torch.zeros(24, KV, page, hd, dtype=DT[dt]) for _ in range(2)]

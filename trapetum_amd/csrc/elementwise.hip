@@ -220,8 +220,9 @@ extern "C" int tp_gather_rows(const float* x, const int* rows, float* out, int n
 // Rotation: pair (d, d + rot/2), angle = pos * inv_freq[d], fp32 cos/sin (runtime/cuda/codebook_gemv.cu:219-230);
 // the cache keeps k after the rotation and v as projected (runtime/src/lib.rs:4487-4490).
 // A sequence's position p lives in row p (or p % rows_cap of a ring), found through its page list.
-// grid (rows, H + KV): block (r, j) rotates query head j, or for j >= H rotates key head j - H and writes it and
-// its value head into the cache straight from registers.
+// grid (rows, groups of heads): a block rotates `hpb` of the row's H + KV heads (query heads first); a thread
+// computes the cosine and sine of its pair once and applies them to all of them.  A key head goes into the
+// cache, with its value head, straight from registers.
 template <typename T>
 __global__ void __launch_bounds__(128)
 rope_kv_write_k(T* __restrict__ q, long q_stride, T* __restrict__ k, long k_stride,
@@ -229,17 +230,15 @@ rope_kv_write_k(T* __restrict__ q, long q_stride, T* __restrict__ k, long k_stri
                 const float* __restrict__ inv_freq, int rot,
                 const int* __restrict__ row_seq, const int* __restrict__ row_pos,
                 const int* __restrict__ new_len, const int* __restrict__ table, int table_w,
-                T* __restrict__ k_pool, T* __restrict__ v_pool, int page, int rows_cap) {
-    const int r = blockIdx.x, j = blockIdx.y;
+                T* __restrict__ k_pool, T* __restrict__ v_pool, int page, int rows_cap, int hpb) {
+    const int r = blockIdx.x;
+    const int j_begin = blockIdx.y * hpb, j_end = min(j_begin + hpb, H + (k ? KV : 0));
     const int pos = row_pos[r];
     const int half = rot / 2;
-    const bool is_q = j < H;
-    if (!is_q && !k) return;
-    T* x = is_q ? q + (size_t)r * q_stride + (size_t)j * hd : k + (size_t)r * k_stride + (size_t)(j - H) * hd;
-    T* kdst = nullptr;
-    T* vdst = nullptr;
-    const T* vsrc = nullptr;
-    if (!is_q) {
+    // where the row's keys and values go: the same page and row for every kv head
+    size_t cache_at = 0;
+    bool cached = false;
+    if (k && j_end > H) {
         const int seq = row_seq[r];
         int row = pos;
         bool keep = true;
@@ -248,30 +247,38 @@ rope_kv_write_k(T* __restrict__ q, long q_stride, T* __restrict__ k, long k_stri
             row = pos % rows_cap;
         }
         const int pg = keep ? table[(size_t)seq * table_w + row / page] : -1;
-        if (pg >= 0) {
-            const size_t off = (((size_t)pg * KV + (j - H)) * page + row % page) * hd;
-            kdst = k_pool + off;
-            vdst = v_pool + off;
-            vsrc = v + (size_t)r * v_stride + (size_t)(j - H) * hd;
-        }
+        cached = pg >= 0;
+        if (cached) cache_at = ((size_t)pg * KV * page + row % page) * hd;      // + kv head * page * hd
     }
     for (int f = threadIdx.x; f < half; f += blockDim.x) {     // one thread per pair (f, f + half)
         const float ang = (float)pos * inv_freq[f];
         const float c = cosf(ang), sn = sinf(ang);
-        const float x0 = ld_f32(x + f), x1 = ld_f32(x + f + half);
-        st_f32(x + f, x0 * c - x1 * sn);
-        st_f32(x + f + half, x1 * c + x0 * sn);
-        if (kdst) {
-            st_f32(kdst + f, x0 * c - x1 * sn);
-            st_f32(kdst + f + half, x1 * c + x0 * sn);
-            vdst[f] = vsrc[f];
-            vdst[f + half] = vsrc[f + half];
+        for (int j = j_begin; j < j_end; j++) {
+            const bool is_q = j < H;
+            T* x = is_q ? q + (size_t)r * q_stride + (size_t)j * hd : k + (size_t)r * k_stride + (size_t)(j - H) * hd;
+            const float x0 = ld_f32(x + f), x1 = ld_f32(x + f + half);
+            const float y0 = x0 * c - x1 * sn, y1 = x1 * c + x0 * sn;
+            st_f32(x + f, y0);
+            st_f32(x + f + half, y1);
+            if (!is_q && cached) {
+                const size_t off = cache_at + (size_t)(j - H) * page * hd;
+                const T* vsrc = v + (size_t)r * v_stride + (size_t)(j - H) * hd;
+                st_f32(k_pool + off + f, y0);
+                st_f32(k_pool + off + f + half, y1);
+                v_pool[off + f] = vsrc[f];
+                v_pool[off + f + half] = vsrc[f + half];
+            }
         }
     }
-    if (kdst)
-        for (int d = rot + threadIdx.x; d < hd; d += blockDim.x) {   // elements outside the rotation
-            kdst[d] = x[d];
-            vdst[d] = vsrc[d];
+    if (cached)
+        for (int j = max(j_begin, H); j < j_end; j++) {           // elements outside the rotation
+            const size_t off = cache_at + (size_t)(j - H) * page * hd;
+            const T* ksrc = k + (size_t)r * k_stride + (size_t)(j - H) * hd;
+            const T* vsrc = v + (size_t)r * v_stride + (size_t)(j - H) * hd;
+            for (int d = rot + threadIdx.x; d < hd; d += blockDim.x) {
+                k_pool[off + d] = ksrc[d];
+                v_pool[off + d] = vsrc[d];
+            }
         }
 }
 
@@ -288,14 +295,17 @@ extern "C" int tp_rope_kv_write(void* q, long q_stride, void* k, long k_stride, 
     TP_REQUIRE(rows_cap >= 0 && (rows_cap == 0 || rows_cap % page == 0), "rope_kv_write: ring of %d rows is no multiple of the page size %d", rows_cap, page);
     hipStream_t s = (hipStream_t)stream;
     TP_REQUIRE(H + KV <= 65535, "rope_kv_write: %d heads exceed one launch", H + KV);
-    dim3 grid(M, H + (k ? KV : 0));
+    // many rows: one block per row shares each pair's cosine and sine over all heads; few rows: a block per head
+    const int heads = H + (k ? KV : 0);
+    const int hpb = M >= 256 ? heads : (M >= 32 ? (heads + 3) / 4 : 1);
+    dim3 grid(M, (heads + hpb - 1) / hpb);
     const int threads = hd <= 64 ? 64 : 128;
     if (dtype == TP_BF16)
         rope_kv_write_k<bf16_t><<<grid, threads, 0, s>>>((bf16_t*)q, q_stride, (bf16_t*)k, k_stride, (const bf16_t*)v, v_stride, H, KV, hd,
-            inv_freq, rot, row_seq, row_pos, new_len, table, table_w, (bf16_t*)k_pool, (bf16_t*)v_pool, page, rows_cap);
+            inv_freq, rot, row_seq, row_pos, new_len, table, table_w, (bf16_t*)k_pool, (bf16_t*)v_pool, page, rows_cap, hpb);
     else if (dtype == TP_F32)
         rope_kv_write_k<float><<<grid, threads, 0, s>>>((float*)q, q_stride, (float*)k, k_stride, (const float*)v, v_stride, H, KV, hd,
-            inv_freq, rot, row_seq, row_pos, new_len, table, table_w, (float*)k_pool, (float*)v_pool, page, rows_cap);
+            inv_freq, rot, row_seq, row_pos, new_len, table, table_w, (float*)k_pool, (float*)v_pool, page, rows_cap, hpb);
     else return tp_fail("rope_kv_write: unknown dtype %d", dtype);
     return tp_check_launch("rope_kv_write");
 }
