@@ -13,6 +13,7 @@ struct GemmArgs {
     int units;              // gated: columns of the output (the feed-forward width)
     void* workspace; size_t workspace_bytes;
     int defer;              // split products: leave the K slices in the workspace [slices, M, N] for the consumer to add
+    int algo;               // the caller's choice of kernel (0: none); 6 asks the tiled kernel for its wide tile
     hipStream_t stream;
 };
 

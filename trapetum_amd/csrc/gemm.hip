@@ -90,11 +90,11 @@ static int check_args(const GemmArgs& a) {
     return 0;
 }
 
-// algo: 0 = choose, 1 = plain, 2 = skinny matrix-core, 3 = tiled matrix-core, 4 = tiled with direct loads
+// algo: 0 = choose, 1 = plain, 2 = skinny matrix-core, 3 = tiled matrix-core (6: with its wide tile), 4 = tiled with direct loads
 static int pick(const GemmArgs& a, int algo) {
     if (algo == 1) return 1;
     if (algo == 2) return gemm_skinny_supports(a) ? 2 : -2;
-    if (algo == 3) return gemm_mfma_supports(a) ? 3 : -3;
+    if (algo == 3 || algo == 6) return gemm_mfma_supports(a) ? 3 : -3;
     if (algo == 4) return gemm_tiled_supports(a) ? 4 : -4;
     // measured on MI355X: from 8 rows on, a very wide product (the logits) streams faster through the tiled
     // kernel's coalesced loads (5.3 TB/s) than through the skinny kernel (4.1 TB/s and falling with the rows)
@@ -108,7 +108,7 @@ static int pick(const GemmArgs& a, int algo) {
 // product comes back as that many K slices
 extern "C" long tp_linear_workspace_bytes(int in_dtype, int out_dtype, int M, int N, int K, int epilogue, int units,
                                           int defer, int algo) {
-    GemmArgs a{nullptr, nullptr, nullptr, in_dtype, out_dtype, M, N, K, epilogue, 1.f, units, nullptr, 0, defer, nullptr};
+    GemmArgs a{nullptr, nullptr, nullptr, in_dtype, out_dtype, M, N, K, epilogue, 1.f, units, nullptr, 0, defer, algo, nullptr};
     const int p = pick(a, algo);
     if (p == 2) return (long)gemm_skinny_workspace(a);
     if (p == 3) { const int s = gemm_mfma_splits(a); return s > 1 ? (long)s * M * N * 4 : 0; }
@@ -120,7 +120,7 @@ extern "C" int tp_linear(const void* x, const void* w, void* y, int in_dtype, in
                          int epilogue, float cap, int units, void* workspace, long workspace_bytes, int defer,
                          int algo, void* stream) {
     GemmArgs a{x, w, y, in_dtype, out_dtype, M, N, K, epilogue, cap, units, workspace, (size_t)workspace_bytes, defer,
-               (hipStream_t)stream};
+               algo, (hipStream_t)stream};
     if (int rc = check_args(a)) return rc;
     const int p = pick(a, algo);
     TP_REQUIRE(p > 0, "linear: the requested kernel (%d) does not take M=%d N=%d K=%d dtype %d", algo, M, N, K, in_dtype);
