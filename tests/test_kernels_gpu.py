@@ -95,13 +95,11 @@ LINEAR_SHAPES = [(1, 16, 8), (3, 100, 72), (17, 331, 88), (64, 130, 2304), (5, 2
 LINEAR_SHAPES += [(65, 100, 64), (300, 257, 576), (1000, 520, 192), (513, 2304, 2048)]
 
 
-@pytest.mark.parametrize("algo", [1, 2, 3, 4, 6])
+@pytest.mark.parametrize("algo", [1, 2, 3, 6])
 @pytest.mark.parametrize("m,n,k", LINEAR_SHAPES)
 def test_linear_bf16(ops, algo, m, n, k):
     if algo == 2 and m > 64:
         pytest.skip("the skinny kernel takes at most 64 rows")
-    if algo == 4 and (m <= 64 or k % 64):
-        pytest.skip("the direct-load kernel takes more than 64 rows and K a multiple of 64")
     x, w = randn(m, k, dtype=torch.bfloat16, seed=7), randn(n, k, dtype=torch.bfloat16, seed=8, scale=0.05)
     ops.force_linear = algo
     try:
@@ -127,7 +125,7 @@ def test_linear_f32(ops, m, n, k):
     assert torch.equal(alone[0], got[m - 1])
 
 
-@pytest.mark.parametrize("algo", [1, 2, 3, 4, 6])
+@pytest.mark.parametrize("algo", [1, 2, 3, 6])
 @pytest.mark.parametrize("dt", ["bf16", "f32"])
 @pytest.mark.parametrize("m,inter,k", [(1, 16, 16), (4, 200, 88), (40, 320, 96), (9, 1000, 2304), (150, 72, 136),
                                        (150, 72, 128), (700, 1000, 320)])
@@ -136,8 +134,6 @@ def test_gated_linear(ops, algo, dt, m, inter, k):
         pytest.skip("float32 runs on the plain kernel only")
     if algo == 2 and m > 64:
         pytest.skip("the skinny kernel takes at most 64 rows")
-    if algo == 4 and (m <= 64 or k % 64):
-        pytest.skip("the direct-load kernel takes more than 64 rows and K a multiple of 64")
     wg, wu = randn(inter, k, dtype=DT[dt], seed=11, scale=0.2), randn(inter, k, dtype=DT[dt], seed=12, scale=0.2)
     x = randn(m, k, dtype=DT[dt], seed=13)
     packed = ops.pack_gate_up(wg, wu)

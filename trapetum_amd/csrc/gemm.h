@@ -26,6 +26,3 @@ int gemm_skinny_launch(const GemmArgs& a);
 bool gemm_mfma_supports(const GemmArgs& a);
 int gemm_mfma_splits(const GemmArgs& a);
 int gemm_mfma_launch(const GemmArgs& a);
-// the same with 256 x 256 tiles and direct loads into LDS; K a multiple of 64
-bool gemm_tiled_supports(const GemmArgs& a);
-int gemm_tiled_launch(const GemmArgs& a);

@@ -90,12 +90,11 @@ static int check_args(const GemmArgs& a) {
     return 0;
 }
 
-// algo: 0 = choose, 1 = plain, 2 = skinny matrix-core, 3 = tiled matrix-core (6: with its wide tile), 4 = tiled with direct loads
+// algo: 0 = choose, 1 = plain, 2 = skinny matrix-core, 3 = tiled matrix-core (6: with its wide tile)
 static int pick(const GemmArgs& a, int algo) {
     if (algo == 1) return 1;
     if (algo == 2) return gemm_skinny_supports(a) ? 2 : -2;
     if (algo == 3 || algo == 6) return gemm_mfma_supports(a) ? 3 : -3;
-    if (algo == 4) return gemm_tiled_supports(a) ? 4 : -4;
     // measured on MI355X: from 8 rows on, a very wide product (the logits) streams faster through the tiled
     // kernel's coalesced loads (5.3 TB/s) than through the skinny kernel (4.1 TB/s and falling with the rows)
     if (a.M >= 8 && a.N >= 32768 && gemm_mfma_supports(a)) return 3;
@@ -126,6 +125,5 @@ extern "C" int tp_linear(const void* x, const void* w, void* y, int in_dtype, in
     TP_REQUIRE(p > 0, "linear: the requested kernel (%d) does not take M=%d N=%d K=%d dtype %d", algo, M, N, K, in_dtype);
     if (p == 2) return gemm_skinny_launch(a);
     if (p == 3) return gemm_mfma_launch(a);
-    if (p == 4) return gemm_tiled_launch(a);
     return gemm_simple_launch(a);
 }

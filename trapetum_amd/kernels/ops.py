@@ -85,7 +85,7 @@ class HipOps:
             raise KernelError(f"the HIP kernel library could not be built or loaded: {e}") from None
         _bind(self.lib, _CORE_SIGS)
         self._attn = {}
-        self.force_linear = 0           # tests: 1 plain, 2 skinny, 3 tiled (6: its wide tile), 4 tiled with direct loads
+        self.force_linear = 0           # tests: 1 plain, 2 skinny, 3 tiled (6: its wide tile)
         self.force_plain_attention = False
 
     # ---- helpers -----------------------------------------------------------------------------------
