@@ -432,10 +432,17 @@ attn_decode_k(DecodeArgs a) {
     if (a.qkv) {
         const int half = a.rot >> 1, rest = HD - a.rot;
         auto val = [&](long col) -> float {
-            if (a.qkv_f32) {
+            if (a.qkv_f32) {                     // slices added in order, four loads in flight at a time
                 const float* src = (const float*)a.qkv + (size_t)seq * a.row_stride + col;
-                float t = src[0];
-                for (int sl = 1; sl < a.n_slices; sl++) t += src[(size_t)sl * a.slice_stride];
+                float t = 0.f;
+                for (int s0 = 0; s0 < a.n_slices; s0 += 4) {
+                    float part[4];
+#pragma unroll
+                    for (int u = 0; u < 4; u++)
+                        part[u] = src[(size_t)(s0 + u < a.n_slices ? s0 + u : a.n_slices - 1) * a.slice_stride];
+#pragma unroll
+                    for (int u = 0; u < 4; u++) t += s0 + u < a.n_slices ? part[u] : 0.f;
+                }
                 return t;
             }
             return bf16_to_f32(((const bf16_t*)a.qkv)[(size_t)seq * a.row_stride + col]);

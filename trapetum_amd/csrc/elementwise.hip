@@ -137,8 +137,21 @@ add_rms_norm_reg_k(float* __restrict__ stream, const TR* __restrict__ rows, int 
     for (int j = 0; j < EPT; j++) {
         const int i = threadIdx.x + j * NTH;
         const bool ok = i < D;
-        a[j] = ok ? ld_f32(ar + i) : 0.f;
-        for (int sl = 1; sl < n_slices; sl++) a[j] += ok ? ld_f32(ar + (size_t)sl * slice_stride + i) : 0.f;
+        // K slices: four loads in flight at a time (a loop of load-then-add would pay one memory round trip per
+        // slice), added in slice order; past the last slice the load repeats it and adds nothing
+        const int ic = ok ? i : 0;
+        float sum = n_slices == 1 ? ld_f32(ar + ic) : 0.f;
+        for (int s0 = 0; s0 < n_slices && n_slices > 1; s0 += 4) {
+            float t[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int sl = s0 + u < n_slices ? s0 + u : n_slices - 1;
+                t[u] = ld_f32(ar + (size_t)sl * slice_stride + ic);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++) sum += s0 + u < n_slices ? t[u] : 0.f;
+        }
+        a[j] = ok ? sum : 0.f;
         v[j] = ok ? sr[i] : 0.f;
         gp[j] = (ok && gain_post) ? gain_post[i] : 1.f;
         gn[j] = (ok && gain_next) ? gain_next[i] : 0.f;
