@@ -82,3 +82,21 @@ def test_unequal_batches_reused_slots(setup):
             ref = plain.forward(pcfg, pw, seqs[i][:n])[lens[i] - 1:n]
             assert rel_l2(torch.stack(got[i]), ref) < tol, (batch, i)
     assert cache.live_slots() == []
+
+
+def test_steps_repeat_bit_for_bit(setup):
+    """The same prefill and the same decode steps, run twice on fresh slots, give the same bits: every reduction has a
+    fixed order (no atomics), whatever the timing of the blocks (runtime/src/lib.rs:1433-1457 checks the same)."""
+    model, cfg, pcfg, pw, tol = setup
+    lens = [41, 7, 23]
+    seqs = [random_tokens(n + 6, cfg.vocab_size, 30 + i) for i, n in enumerate(lens)]
+    runs = []
+    for _ in range(2):
+        cache = model.new_cache(max_tokens=512, page_size=16)
+        slots = [cache.acquire() for _ in lens]
+        flat = [t for s, n in zip(seqs, lens) for t in s[:n]]
+        rows = [model.step(cache, slots, flat, counts=lens, want=list(range(sum(lens))))]
+        for step in range(6):
+            rows.append(model.step(cache, slots, [s[n + step] for s, n in zip(seqs, lens)]))
+        runs.append(torch.cat(rows).cpu())
+    assert torch.equal(runs[0], runs[1])

@@ -342,3 +342,43 @@ def test_argmax_ties_and_nan(ops):
     assert ops.argmax(z.to(DEV)).tolist() == [100, 7000, 5]
     big = randn(5, 256000, seed=60)
     assert ops.argmax(big).tolist() == big.cpu().argmax(dim=-1).tolist()
+
+
+# ---- token choice ----------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("vocab,temperature,top_k,top_p", [(256, 0.7, 256, 0.95), (7001, 1.0, 40, 1.0), (7001, 0.3, 1000, 0.5),
+                                                           (256000, 0.9, 256, 0.95), (513, 1.5, 1, 1.0), (513, 0.8, 600, 0.99)])
+def test_sample_follows_the_plain_sampler(ops, vocab, temperature, top_k, top_p):
+    """Sort by logit (ties: smaller id), keep top_k, softmax at the temperature, shortest prefix reaching top_p, walk
+    with u (runtime/src/bin/serve.rs:41-72).  Ties and a dominant token are planted; where the uniform number falls
+    within float32 rounding of a boundary of the walk either neighbour is right."""
+    rows = 6
+    z = randn(rows, vocab, seed=80, scale=3.0).cpu()
+    z[1, 5] = z[1, 77] = z[1].max() + 1.0                    # a tie at the top
+    z[2, vocab - 1] = z[2].max() + 30.0                      # one token takes all the mass
+    u = torch.tensor([0.0, 0.5, 0.999, 0.25, 0.75, 0.9999], dtype=torch.float32)
+    with pytest.raises(Exception, match="top_k"):            # the kernel sorts at most 1024 candidates and says so
+        ops.sample(z.to(DEV), temperature, 2000, top_p, u.to(DEV))
+    got = ops.sample(z.to(DEV), temperature, top_k, top_p, u.to(DEV)).cpu().tolist()
+    for b in range(rows):
+        choices = set()
+        for du in (-2e-6, 0.0, 2e-6):
+            ub = min(max(float(u[b]) + du, 0.0), 0.9999999)
+            choices.add(int(ref_ops.sample(z[b:b + 1], temperature, top_k, top_p, torch.tensor([ub]))[0]))
+        assert got[b] in choices, (b, got[b], choices)
+    assert got[2] == vocab - 1
+
+
+@pytest.mark.parametrize("vocab,window", [(256, 8), (256000, 128)])
+def test_repetition_penalty(ops, vocab, window):
+    """Each distinct recent token once: z / penalty if z > 0 else z * penalty (runtime/src/bin/serve.rs:1330-1340)."""
+    z = randn(3, vocab, seed=81, scale=2.0)
+    recent = torch.full((3, window), -1, dtype=torch.int32)
+    recent[0, :4] = torch.tensor([3, 3, 9, vocab - 1])       # a token twice in the window is penalised once
+    recent[1, :] = torch.arange(window) * 2 % vocab
+    ref = z.cpu().clone()
+    ref_ops.apply_repetition_penalty(ref, recent, 1.3)
+    ops.apply_repetition_penalty(z, recent.to(DEV), 1.3)
+    assert torch.allclose(z.cpu(), ref, rtol=1e-6, atol=0)
+    untouched = z.cpu().clone()
+    ops.apply_repetition_penalty(z, recent.to(DEV), 1.0)     # 1.0 switches it off
+    assert torch.equal(z.cpu(), untouched)
