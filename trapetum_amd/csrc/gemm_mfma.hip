@@ -127,21 +127,36 @@ bool gemm_mfma_supports(const GemmArgs& a) {
     return a.in_dtype == TP_BF16 && a.K % 8 == 0;
 }
 
-// Tile of a product: 128 x 256 (less LDS traffic per matrix instruction; two blocks fit a CU) where the grid is at
-// least four rounds of those 512 places, so that a last, partly filled round costs little; else 128 x 128 (three
-// blocks a CU).  Measured on the 2B gate/up product: 930 against 790 TFLOP/s at 8192 rows, 700 against 790 at 2048.
-static bool wide_tile(const GemmArgs& a) {
-    return a.algo == 6 || (long)tp_cdiv(a.M, 128) * tp_cdiv(a.N, 256) >= 2048;
+// Tile of a product, in 16 x 16 tiles of a wave (the block is 2 x 2 waves).  Up to 64 rows: 64 x 64, the most
+// blocks per byte of W.  Else 128 x 256 (less LDS traffic per matrix instruction; two blocks fit a CU) where the grid
+// is at least four rounds of those 512 places, so that a last, partly filled round costs little; else 128 x 128
+// (three blocks a CU).  Measured on the 2B gate/up product: 930 against 790 TFLOP/s at 8192 rows, 700 against 790
+// at 2048; at 64 rows 35 us with 64 x 64 tiles against 45 us with 128 x 128.
+struct Tile { int tm, tn; };
+static Tile pick_tile(const GemmArgs& a) {
+    if (a.algo == 6) return {4, 8};
+    if (a.M <= 64 && !(a.M > 32 && a.N >= 32768)) return {2, 2};    // the logits of 64 rows: 250 us with 128 x 128, 275 with 64 x 64
+    if ((long)tp_cdiv(a.M, 128) * tp_cdiv(a.N, 256) >= 2048) return {4, 8};
+    return {4, 4};
 }
 
 // K slices for products whose tiles alone do not fill the chip and whose consumer adds the slices (defer)
 int gemm_mfma_splits(const GemmArgs& a) {
     if (!a.defer || a.epilogue != TP_EPI_NONE || a.algo == 6) return 1;
-    const long blocks = (long)tp_cdiv(a.M, 128) * tp_cdiv(a.N, 128);
-    if (blocks >= 448 || a.K < 1024) return 1;          // measured at 288 tiles: the slices win back a fifth
-    int s = (int)(640 / blocks);
-    if (s > a.K / 512) s = a.K / 512;
-    if (s > 4) s = 4;
+    const Tile t = pick_tile(a);
+    const long blocks = (long)tp_cdiv(a.M, 32 * t.tm) * tp_cdiv(a.N, 32 * t.tn);
+    int s;
+    if (t.tm == 2) {                                    // few rows: bound by reading W, wants every CU streaming
+        if (blocks >= 512 || a.K < 512) return 1;
+        s = (int)tp_cdiv(640, blocks);
+        if (s > a.K / 256) s = a.K / 256;
+        if (s > 16) s = 16;
+    } else {
+        if (blocks >= 448 || a.K < 1024) return 1;      // measured at 288 tiles: the slices win back a fifth
+        s = (int)(640 / blocks);
+        if (s > a.K / 512) s = a.K / 512;
+        if (s > 4) s = 4;
+    }
     return s < 1 ? 1 : s;
 }
 
@@ -153,28 +168,28 @@ static void mfma_launch(const GemmArgs& a, void* y, int out_dtype, int splits, i
                                                          out_dtype, a.cap, a.units, kps);
 }
 
+template <int EPI>
+static void mfma_launch_tile(const GemmArgs& a, Tile t, void* y, int out_dtype, int splits, int kps) {
+    if (t.tm == 2) mfma_launch<EPI, 2, 2>(a, y, out_dtype, splits, kps);
+    else if (t.tn == 8) mfma_launch<EPI, 4, 8>(a, y, out_dtype, splits, kps);
+    else mfma_launch<EPI, 4, 4>(a, y, out_dtype, splits, kps);
+}
+
 int gemm_mfma_launch(const GemmArgs& a) {
     TP_REQUIRE(gemm_mfma_supports(a), "tiled product: needs bf16 and K a multiple of 8 (K=%d)", a.K);
     TP_REQUIRE(((uintptr_t)a.x % 16 == 0) && ((uintptr_t)a.w % 16 == 0), "tiled product: operands must be 16-byte aligned");
-    TP_REQUIRE((long)tp_cdiv(a.M, 128) * tp_cdiv(a.N, 128) < (1L << 31), "tiled product: too many tiles for one launch (M=%d N=%d)", a.M, a.N);
+    TP_REQUIRE((long)tp_cdiv(a.M, 64) * tp_cdiv(a.N, 64) < (1L << 31), "tiled product: too many tiles for one launch (M=%d N=%d)", a.M, a.N);
+    const Tile t = pick_tile(a);
     const int splits = gemm_mfma_splits(a);
     if (splits > 1) {
         const size_t need = (size_t)splits * a.M * a.N * sizeof(float);
         TP_REQUIRE(a.workspace && a.workspace_bytes >= need, "tiled product: workspace of %zu bytes, %zu needed", a.workspace_bytes, need);
         const int kps = tp_cdiv(tp_cdiv(a.K, splits), BK) * BK;
-        mfma_launch<TP_EPI_NONE, 4, 4>(a, a.workspace, TP_F32, tp_cdiv(a.K, kps), kps);
+        mfma_launch_tile<TP_EPI_NONE>(a, t, a.workspace, TP_F32, tp_cdiv(a.K, kps), kps);
         return tp_check_launch("linear (tiled kernel, K slices)");
     }
-    const bool wide = wide_tile(a);
-    if (a.epilogue == TP_EPI_GATED) {
-        if (wide) mfma_launch<TP_EPI_GATED, 4, 8>(a, a.y, a.out_dtype, 1, a.K);
-        else mfma_launch<TP_EPI_GATED, 4, 4>(a, a.y, a.out_dtype, 1, a.K);
-    } else if (a.epilogue == TP_EPI_SOFTCAP) {
-        if (wide) mfma_launch<TP_EPI_SOFTCAP, 4, 8>(a, a.y, a.out_dtype, 1, a.K);
-        else mfma_launch<TP_EPI_SOFTCAP, 4, 4>(a, a.y, a.out_dtype, 1, a.K);
-    } else {
-        if (wide) mfma_launch<TP_EPI_NONE, 4, 8>(a, a.y, a.out_dtype, 1, a.K);
-        else mfma_launch<TP_EPI_NONE, 4, 4>(a, a.y, a.out_dtype, 1, a.K);
-    }
+    if (a.epilogue == TP_EPI_GATED) mfma_launch_tile<TP_EPI_GATED>(a, t, a.y, a.out_dtype, 1, a.K);
+    else if (a.epilogue == TP_EPI_SOFTCAP) mfma_launch_tile<TP_EPI_SOFTCAP>(a, t, a.y, a.out_dtype, 1, a.K);
+    else mfma_launch_tile<TP_EPI_NONE>(a, t, a.y, a.out_dtype, 1, a.K);
     return tp_check_launch("linear (tiled kernel)");
 }
