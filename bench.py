@@ -1,6 +1,7 @@
 """Benchmark: decode tokens per second of Gemma-2 at 2B layer sizes with random weights on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--dtype bfloat16|float32]
+                    [--sizes 2b|9b|27b] [--prompt T]
 
 A step is one decode step of a batch of 8 sequences (a token each, chosen greedily on the device and fed to
 the next step).  One JSON line is printed: decode tokens per second as `value`, the prefill of 2,048 tokens,
@@ -21,7 +22,13 @@ SIZES = dict(num_hidden_layers=26, hidden_size=2304, num_attention_heads=8, num_
              intermediate_size=9216, vocab_size=256000, rms_norm_eps=1e-6, rope_theta=10000.0, sliding_window=4096,
              query_pre_attn_scalar=256, attn_logit_softcapping=50.0, final_logit_softcapping=30.0,
              max_position_embeddings=8192)
-FULL_LAYERS = SIZES["num_hidden_layers"]
+# the other two Gemma-2 sizes, for `--sizes`: what differs from the 2B configuration
+OTHER_SIZES = {
+    "2b": {},
+    "9b": dict(num_hidden_layers=42, hidden_size=3584, num_attention_heads=16, num_key_value_heads=8, intermediate_size=14336),
+    "27b": dict(num_hidden_layers=46, hidden_size=4608, num_attention_heads=32, num_key_value_heads=16, head_dim=128,
+                intermediate_size=36864, query_pre_attn_scalar=144),
+}
 CONTEXT, PROMPT, PREFILL_TOKENS, BATCH = 8192, 512, 2048, 8
 
 
@@ -56,7 +63,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)
-    ap.add_argument("--layers", type=int, default=FULL_LAYERS, help="fewer layers than the configuration's, if memory or time needs it")
+    ap.add_argument("--sizes", default="2b", choices=sorted(OTHER_SIZES), help="layer sizes of which Gemma-2 (the metric is 2b)")
+    ap.add_argument("--layers", type=int, default=0, help="fewer layers than the configuration's, if memory or time needs it")
+    ap.add_argument("--prompt", type=int, default=PROMPT, help="tokens of each prompt before decoding (the metric: 512)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
     ap.add_argument("--no-graph", action="store_true", help="launch decode steps kernel by kernel instead of replaying a HIP graph")
@@ -71,11 +80,14 @@ def main():
     from trapetum_amd.engine import Engine
     from trapetum_amd.engine.decode_loop import DecodeLoop
 
-    cfg = Gemma2Config.from_kwargs(**dict(SIZES, num_hidden_layers=args.layers))
+    sizes = dict(SIZES, **OTHER_SIZES[args.sizes])
+    full_layers = sizes["num_hidden_layers"]
+    cfg = Gemma2Config.from_kwargs(**dict(sizes, num_hidden_layers=args.layers or full_layers))
     itemsize = 2 if args.dtype == "bfloat16" else 4
     t0 = time.time()
+    most = max(PREFILL_TOKENS, (BATCH if args.no_points else 64) * (args.prompt + args.steps + args.warmup + 128))
     engine = Engine.from_config(cfg, seed=2, sigma=0.02, dtype=args.dtype, draw_on_device=True,
-                                max_tokens_in_cache=64 * 1024, max_context=CONTEXT, max_batch=64)
+                                max_tokens_in_cache=max(64 * 1024, most), max_context=CONTEXT, max_batch=64)
     model, cache = engine.model, engine.cache
     torch.cuda.synchronize()
     print(f"[bench] model ready in {time.time() - t0:.1f}s", file=sys.stderr, flush=True)
@@ -105,11 +117,11 @@ def main():
     # ---- decode ---------------------------------------------------------------------------------------------
     def decode(batch, steps, warmup):
         loop = DecodeLoop(model, cache, use_graph=not args.no_graph)
-        loop.start(prompts(batch, PROMPT))
+        loop.start(prompts(batch, args.prompt))
         for _ in range(warmup):
             loop.step()
         torch.cuda.synchronize()
-        ctx0 = PROMPT + warmup
+        ctx0 = args.prompt + warmup
         t = time.perf_counter()
         for _ in range(steps):
             loop.step()
@@ -133,14 +145,14 @@ def main():
             print(f"[bench] decode batch {b}: {points[f'decode_b{b}']} tok/s", file=sys.stderr, flush=True)
 
     line = {
-        "metric": "decode tok/s @ batch 8, Gemma-2-2B layer sizes", "value": round(value, 1), "unit": "tok/s",
+        "metric": f"decode tok/s @ batch 8, Gemma-2-{args.sizes.upper()} layer sizes", "value": round(value, 1), "unit": "tok/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
         "data": "synthetic: seeded random weights N(0, 0.02) and uniform-random token ids",
-        "config": {"model": "gemma-2-2b sizes", "layers": args.layers, "layers_full": FULL_LAYERS,
+        "config": {"model": f"gemma-2-{args.sizes} sizes", "layers": cfg.num_hidden_layers, "layers_full": full_layers,
                    "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
                    "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
-                   "window": cfg.sliding_window, "global_batch": BATCH, "seq_len": CONTEXT, "prompt_len": PROMPT,
+                   "window": cfg.sliding_window, "global_batch": BATCH, "seq_len": CONTEXT, "prompt_len": args.prompt,
                    "decode_context": round(mean_ctx, 1), "hip_graph": not args.no_graph, "parallelism": "single GPU"},
         "prefill": prefill, "roofline": roofline, "points": points,
     }
