@@ -101,3 +101,27 @@ def test_graph_replays_equal_eager_steps(folders):
     for step in range(12, 16):
         step_toks = [toks[i][lens[i] + step] for i in range(2)]
         assert torch.equal(model.step(eager_cache, es, step_toks), graphed.step(gs, step_toks)), step
+
+
+def test_graphs_follow_a_sequence_across_their_length_bound(folders):
+    """A graph serves lengths up to a bound (1024, 2048, ...); a sequence that grows past it moves to the next graph.
+    Replays before, at and after the crossing agree with eager steps (the slices of the keys differ, so to rounding)."""
+    from .gpu_engine import load_gpu_model
+    from trapetum_amd.engine.graphs import GraphedDecode
+    model, cfg = load_gpu_model(folders["B"], "bfloat16")
+    lens = [1015, 300]
+    toks = [random_tokens(n + 24, cfg.vocab_size, 90 + i) for i, n in enumerate(lens)]
+    eager_cache = model.new_cache(max_tokens=4096)
+    graph_cache = model.new_cache(max_tokens=4096)
+    graphed = GraphedDecode(model, graph_cache)
+    es = [eager_cache.acquire() for _ in toks]
+    gs = [graph_cache.acquire() for _ in toks]
+    flat = [t for s, n in zip(toks, lens) for t in s[:n]]
+    model.step(eager_cache, es, flat, counts=lens)
+    model.step(graph_cache, gs, flat, counts=lens)
+    for step in range(24):
+        step_toks = [toks[i][lens[i] + step] for i in range(2)]
+        a = model.step(eager_cache, es, step_toks).clone()
+        b = graphed.step(gs, step_toks).clone()
+        assert rel_l2(b, a) < 3e-3, step
+    assert len(graphed.by_batch) == 2
