@@ -129,7 +129,7 @@ extern "C" int tp_repetition_penalty(float* logits, int B, int V, const int* rec
 // p = exp((z - max) / T) / sum, the shortest prefix whose cumulative mass reaches top_p, then a walk with
 // r = u * kept mass; falls back to the first candidate.  One block per row: a radix select over the value
 // bits finds the k-th largest logit, an id select breaks ties at that value, the at most 1024 candidates are
-// sorted in LDS, and one thread does the short sequential part in the reference's order of additions. -------
+// sorted in LDS, and the first wave does the short scans (sums in candidate order within a lane, then over the lanes). ---
 __device__ __forceinline__ uint32_t value_key(float f) {           // larger float -> larger key; NaN lowest
     uint32_t u = __float_as_uint(f);
     if ((u & 0x7fffffffu) > 0x7f800000u) return 0u;
@@ -140,9 +140,55 @@ __device__ __forceinline__ float key_value(uint32_t k) {
     return __uint_as_float(u);
 }
 
+// ---- the sampler's short scans, done by the block's first wave (a single thread walking LDS pays its latency per
+// element: 45 us for 256 candidates) -----------------------------------------------------------------------------
+__device__ __forceinline__ unsigned wave_scan_incl(unsigned v, int lane) {
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const unsigned t = (unsigned)__shfl_up((int)v, o, 64);
+        if (lane >= o) v += t;
+    }
+    return v;
+}
+__device__ __forceinline__ float wave_scan_incl(float v, int lane) {
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const float t = __shfl_up(v, o, 64);
+        if (lane >= o) v += t;
+    }
+    return v;
+}
+// Walks the 256 counters from the top (or from the bottom) until `rem` of them are covered: the bucket that holds the
+// rem-th member, and how many of that bucket are still needed.  All 64 lanes of one wave call it.
+__device__ __forceinline__ void pick_bucket(const unsigned* hist, bool from_top, unsigned rem, int lane, int& bucket, unsigned& rem_out) {
+    unsigned c[4], local = 0u;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int o = lane * 4 + j;
+        c[j] = hist[from_top ? 255 - o : o];
+        local += c[j];
+    }
+    const unsigned incl = wave_scan_incl(local, lane);
+    const unsigned long long hit = __ballot(incl >= rem);
+    const int L = hit ? __ffsll((long long)hit) - 1 : 63;
+    unsigned r = rem - (incl - local);
+    int j = 0;
+    for (; j < 3; j++) {
+        if (c[j] >= r) break;
+        r -= c[j];
+    }
+    const int o = L * 4 + __shfl(j, L, 64);
+    bucket = from_top ? 255 - o : o;
+    rem_out = (unsigned)__shfl((int)r, L, 64);
+}
+
+// With a candidate list (cand_count non-null): row b's candidates are cand_val/cand_id[b * cand_cap ..], a superset
+// of its top_k if their number fits cand_cap; the kernel then works on the list, else on the whole row.
 __global__ void __launch_bounds__(1024)
 sample_k(const float* __restrict__ logits, int V, float temperature, int top_k, float top_p,
-         const float* __restrict__ uniforms, int* __restrict__ out) {
+         const float* __restrict__ uniforms, int* __restrict__ out,
+         const unsigned* __restrict__ cand_count, const float* __restrict__ cand_val, const int* __restrict__ cand_id,
+         int cand_cap) {
     __shared__ unsigned hist[256];
     __shared__ uint32_t ckey[1024];
     __shared__ int cid[1024];
@@ -151,7 +197,13 @@ sample_k(const float* __restrict__ logits, int V, float temperature, int top_k, 
     __shared__ int s_id_limit;
     const float* z = logits + (size_t)blockIdx.x * V;
     const int tid = threadIdx.x;
-    const int k = top_k < V ? top_k : V;
+    const int k = top_k < V ? top_k : V;                       // of the whole row, whichever source is read
+    const int* ids = nullptr;                                  // candidate -> token id; null: the index is the id
+    if (cand_count && cand_count[blockIdx.x] <= (unsigned)cand_cap && cand_count[blockIdx.x] >= (unsigned)k) {
+        V = (int)cand_count[blockIdx.x];
+        z = cand_val + (size_t)blockIdx.x * cand_cap;
+        ids = cand_id + (size_t)blockIdx.x * cand_cap;
+    }
 
     // 1. the k-th largest value key, 8 bits at a time from the top
     if (tid == 0) { s_prefix = 0u; s_remaining = (unsigned)k; }
@@ -164,16 +216,15 @@ sample_k(const float* __restrict__ logits, int V, float temperature, int top_k, 
             if (shift == 24 || (key >> (shift + 8)) == (prefix >> (shift + 8))) atomicAdd(&hist[(key >> shift) & 255u], 1u);
         }
         __syncthreads();
-        if (tid == 0) {
-            unsigned rem = s_remaining;
-            int b = 255;
-            for (; b > 0; b--) {
-                if (hist[b] >= rem) break;
-                rem -= hist[b];
+        if (tid < 64) {
+            int b;
+            unsigned rem;
+            pick_bucket(hist, true, s_remaining, tid, b, rem);
+            if (tid == 0) {
+                s_prefix = prefix | ((unsigned)b << shift);
+                s_remaining = rem;                   // how many of this bucket are still needed
+                if (shift == 0) s_eq_total = hist[b];
             }
-            s_prefix = prefix | ((unsigned)b << shift);
-            s_remaining = rem;                       // how many of this bucket are still needed
-            if (shift == 0) s_eq_total = hist[b];
         }
         __syncthreads();
     }
@@ -190,19 +241,18 @@ sample_k(const float* __restrict__ logits, int V, float temperature, int top_k, 
             const unsigned prefix = s_prefix;
             for (int i = tid; i < V; i += blockDim.x) {
                 if (value_key(z[i]) != tkey) continue;
-                const unsigned id = (unsigned)i;
+                const unsigned id = (unsigned)(ids ? ids[i] : i);
                 if (shift == 24 || (id >> (shift + 8)) == (prefix >> (shift + 8))) atomicAdd(&hist[(id >> shift) & 255u], 1u);
             }
             __syncthreads();
-            if (tid == 0) {
-                unsigned rem = s_remaining;
-                int b = 0;
-                for (; b < 255; b++) {
-                    if (hist[b] >= rem) break;
-                    rem -= hist[b];
+            if (tid < 64) {
+                int b;
+                unsigned rem;
+                pick_bucket(hist, false, s_remaining, tid, b, rem);
+                if (tid == 0) {
+                    s_prefix = prefix | ((unsigned)b << shift);
+                    s_remaining = rem;
                 }
-                s_prefix = prefix | ((unsigned)b << shift);
-                s_remaining = rem;
             }
             __syncthreads();
         }
@@ -217,9 +267,10 @@ sample_k(const float* __restrict__ logits, int V, float temperature, int top_k, 
     const int id_limit = s_id_limit;
     for (int i = tid; i < V; i += blockDim.x) {
         const uint32_t key = value_key(z[i]);
-        if (key > tkey || (key == tkey && i <= id_limit)) {
+        const int id = ids ? ids[i] : i;
+        if (key > tkey || (key == tkey && id <= id_limit)) {
             const unsigned at = atomicAdd(&s_count, 1u);
-            if (at < 1024u) { ckey[at] = key; cid[at] = i; }
+            if (at < 1024u) { ckey[at] = key; cid[at] = id; }
         }
     }
     __syncthreads();
@@ -237,38 +288,169 @@ sample_k(const float* __restrict__ logits, int V, float temperature, int top_k, 
             __syncthreads();
         }
     }
-    // 5. probabilities, the nucleus and the draw
+    // 5. probabilities, the nucleus and the draw: the first wave, each lane 16 consecutive candidates; sums run over a
+    // lane's candidates in order, then over the lanes in order
     const float mx = key_value(ckey[0]);
     if (tid < k) prob[tid] = expf((key_value(ckey[tid]) - mx) / temperature);
     __syncthreads();
-    if (tid == 0) {
-        float sum = 0.f;
-        for (int j = 0; j < k; j++) sum += prob[j];
-        for (int j = 0; j < k; j++) prob[j] /= sum;
-        float cum = 0.f;
-        int keep = k;
-        for (int j = 0; j < k; j++) {
-            cum += prob[j];
-            if (cum >= top_p) { keep = j + 1; break; }
-        }
-        float kept = 0.f;
-        for (int j = 0; j < keep; j++) kept += prob[j];
-        float r = uniforms[blockIdx.x] * kept;
-        int pick = cid[0];
-        for (int j = 0; j < keep; j++) {
-            if (r < prob[j]) { pick = cid[j]; break; }
-            r -= prob[j];
-        }
-        out[blockIdx.x] = pick;
+    if (tid < 64) {
+        const int j0 = tid * 16;
+        float local = 0.f;
+        for (int j = j0; j < j0 + 16 && j < k; j++) local += prob[j];
+        const float total = __shfl(wave_scan_incl(local, tid), 63, 64);
+        // cumulative probabilities (reusing the key array's space: 1024 floats)
+        float* cum = reinterpret_cast<float*>(ckey);
+        float lsum = 0.f;
+        for (int j = j0; j < j0 + 16 && j < k; j++) { prob[j] /= total; lsum += prob[j]; }
+        float run = wave_scan_incl(lsum, tid) - lsum;
+        for (int j = j0; j < j0 + 16 && j < k; j++) { run += prob[j]; cum[j] = run; }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        // the shortest prefix whose mass reaches top_p
+        int first = k;
+        for (int j = j0; j < j0 + 16 && j < k; j++)
+            if (cum[j] >= top_p) { first = j; break; }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) first = min(first, __shfl_xor(first, o, 64));
+        const int keep = first < k ? first + 1 : k;
+        const float kept = cum[keep - 1];
+        const float r = uniforms[blockIdx.x] * kept;
+        // the walk: the first candidate whose cumulative mass exceeds r; none (rounding at the end): the first candidate
+        int hit = keep;
+        for (int j = j0; j < j0 + 16 && j < keep; j++)
+            if (r < cum[j]) { hit = j; break; }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) hit = min(hit, __shfl_xor(hit, o, 64));
+        if (tid == 0) out[blockIdx.x] = cid[hit < keep ? hit : 0];
     }
 }
 
+// ---- a coarse filter in front of the exact sampler, on many blocks: the sampler alone reads a row of 256,000
+// logits several times on one CU (0.4 ms).  A histogram of the top 12 bits of the value keys gives the bin that
+// holds the top_k-th largest logit; everything from that bin upwards (top_k plus that bin's other members, a few
+// hundred for logits of a language model) is copied to a candidate list, which the sampler then works on.  A list
+// that would not fit falls back to the whole row, so the result never depends on the filter. -------------------
+constexpr int FILTER_BINS = 4096;
+constexpr int FILTER_PART = 8192;                    // logits per block
+
+__global__ void __launch_bounds__(256)
+filter_hist_k(const float* __restrict__ logits, int V, unsigned* __restrict__ hist) {
+    __shared__ unsigned local[FILTER_BINS];
+    for (int i = threadIdx.x; i < FILTER_BINS; i += 256) local[i] = 0u;
+    __syncthreads();
+    const float* z = logits + (size_t)blockIdx.y * V;
+    const int begin = blockIdx.x * FILTER_PART, end = min(V, begin + FILTER_PART);
+    for (int i = begin + threadIdx.x; i < end; i += 256) atomicAdd(&local[value_key(z[i]) >> 20], 1u);
+    __syncthreads();
+    unsigned* row = hist + (size_t)blockIdx.y * FILTER_BINS;
+    for (int i = threadIdx.x; i < FILTER_BINS; i += 256)
+        if (local[i]) atomicAdd(&row[i], local[i]);
+}
+
+// the bin of the k-th largest key; the histogram and the candidate counter are left zeroed for the next call
+__global__ void __launch_bounds__(256)
+filter_bin_k(unsigned* __restrict__ hist, int k, unsigned* __restrict__ bin_out, unsigned* __restrict__ cand_count) {
+    __shared__ unsigned part[256];
+    unsigned* row = hist + (size_t)blockIdx.x * FILTER_BINS;
+    const int tid = threadIdx.x;
+    constexpr int PER = FILTER_BINS / 256;           // thread t owns bins t*PER .. t*PER+PER-1
+    unsigned mine[PER], sum = 0u;
+#pragma unroll
+    for (int j = 0; j < PER; j++) { mine[j] = row[tid * PER + j]; sum += mine[j]; row[tid * PER + j] = 0u; }
+    part[tid] = sum;
+    __syncthreads();
+    if (tid == 0) {
+        unsigned above = 0u;                         // members of the bins above the current thread's
+        int t = 255;
+        for (; t > 0; t--) {
+            if (above + part[t] >= (unsigned)k) break;
+            above += part[t];
+        }
+        part[0] = (unsigned)t;
+        part[1] = above;
+        cand_count[blockIdx.x] = 0u;
+    }
+    __syncthreads();
+    if (tid == (int)part[0]) {
+        unsigned above = part[1];
+        int j = PER - 1;
+        for (; j > 0; j--) {
+            if (above + mine[j] >= (unsigned)k) break;
+            above += mine[j];
+        }
+        bin_out[blockIdx.x] = (unsigned)(tid * PER + j);
+    }
+}
+
+// a block gathers its candidates in LDS and reserves their places with one addition to the row's counter
+__global__ void __launch_bounds__(256)
+filter_collect_k(const float* __restrict__ logits, int V, const unsigned* __restrict__ bin, unsigned* __restrict__ cand_count,
+                 float* __restrict__ cand_val, int* __restrict__ cand_id, int cand_cap) {
+    constexpr int LOCAL = 1024;
+    __shared__ float lval[LOCAL];
+    __shared__ int lid[LOCAL];
+    __shared__ unsigned lcount, base;
+    if (threadIdx.x == 0) lcount = 0u;
+    __syncthreads();
+    const float* z = logits + (size_t)blockIdx.y * V;
+    const unsigned lowest = bin[blockIdx.y];
+    const int begin = blockIdx.x * FILTER_PART, end = min(V, begin + FILTER_PART);
+    for (int i = begin + threadIdx.x; i < end; i += 256) {
+        const float v = z[i];
+        if ((value_key(v) >> 20) >= lowest) {
+            const unsigned at = atomicAdd(&lcount, 1u);
+            if (at < (unsigned)LOCAL) { lval[at] = v; lid[at] = i; }
+        }
+    }
+    __syncthreads();
+    const unsigned n = lcount;
+    if (n == 0u) return;
+    // more than the block can hold: the row's count is pushed past the capacity, and the sampler reads the whole row
+    if (threadIdx.x == 0) base = atomicAdd(&cand_count[blockIdx.y], n <= (unsigned)LOCAL ? n : (unsigned)cand_cap + 1u);
+    __syncthreads();
+    if (n > (unsigned)LOCAL) return;
+    for (unsigned j = threadIdx.x; j < n; j += 256) {
+        const unsigned at = base + j;
+        if (at < (unsigned)cand_cap) {
+            cand_val[(size_t)blockIdx.y * cand_cap + at] = lval[j];
+            cand_id[(size_t)blockIdx.y * cand_cap + at] = lid[j];
+        }
+    }
+}
+
+constexpr int CAND_CAP = 8192;
+
+// bytes of the sampler's workspace for B rows; it must be zero before its first use and is left ready for the next
+extern "C" long tp_sample_workspace_bytes(int B, int V) {
+    if (V < 4 * FILTER_PART) return 0;               // small vocabularies: the sampler alone
+    return (long)B * (FILTER_BINS * 4 + 8 + (long)CAND_CAP * 8);
+}
+
 extern "C" int tp_sample(const float* logits, int B, int V, float temperature, int top_k, float top_p,
-                         const float* uniforms, int* out, void* stream) {
+                         const float* uniforms, int* out, void* workspace, void* stream) {
     TP_REQUIRE(B > 0 && V > 0, "sample: empty shape B=%d V=%d", B, V);
     TP_REQUIRE(temperature > 0.f, "sample: temperature %g must be positive (0 means argmax)", temperature);
     TP_REQUIRE(top_k >= 1 && top_k <= 1024, "sample: top_k %d must lie in 1..1024", top_k);
     TP_REQUIRE(top_p > 0.f, "sample: top_p %g must be positive", top_p);
-    sample_k<<<B, 1024, 0, (hipStream_t)stream>>>(logits, V, temperature, top_k, top_p, uniforms, out);
+    TP_REQUIRE(B <= 65535, "sample: %d rows exceed one launch", B);
+    hipStream_t s = (hipStream_t)stream;
+    if (!workspace || tp_sample_workspace_bytes(B, V) == 0) {
+        sample_k<<<B, 1024, 0, s>>>(logits, V, temperature, top_k, top_p, uniforms, out, nullptr, nullptr, nullptr, 0);
+        return tp_check_launch("sample");
+    }
+    unsigned* hist = (unsigned*)workspace;
+    unsigned* bin = hist + (size_t)B * FILTER_BINS;
+    unsigned* count = bin + B;
+    float* cand_val = (float*)(count + B);
+    int* cand_id = (int*)(cand_val + (size_t)B * CAND_CAP);
+    const dim3 grid(tp_cdiv(V, FILTER_PART), B);
+    filter_hist_k<<<grid, 256, 0, s>>>(logits, V, hist);
+    if (int rc = tp_check_launch("sample (histogram)")) return rc;
+    filter_bin_k<<<B, 256, 0, s>>>(hist, top_k < V ? top_k : V, bin, count);
+    if (int rc = tp_check_launch("sample (threshold bin)")) return rc;
+    filter_collect_k<<<grid, 256, 0, s>>>(logits, V, bin, count, cand_val, cand_id, CAND_CAP);
+    if (int rc = tp_check_launch("sample (candidates)")) return rc;
+    sample_k<<<B, 1024, 0, s>>>(logits, V, temperature, top_k, top_p, uniforms, out, count, cand_val, cand_id, CAND_CAP);
     return tp_check_launch("sample");
 }

@@ -27,7 +27,8 @@ _CORE_SIGS = {
     "tp_argmax": [_P, _I, _I, _P, _P, _P],
     "tp_argmax_workspace_bytes": [_I, _I],
     "tp_repetition_penalty": [_P, _I, _I, _P, _I, _F, _P],
-    "tp_sample": [_P, _I, _I, _F, _I, _F, _P, _P, _P],
+    "tp_sample": [_P, _I, _I, _F, _I, _F, _P, _P, _P, _P],
+    "tp_sample_workspace_bytes": [_I, _I],
 }
 _ATTN_SIGS = {
     "tp_attn_prefill": [_P, _L, _P, _L, _P, _L, _I, _I, _I, _P, _I, _I, _F, _F, _I, _P, _P, _P],
@@ -85,6 +86,7 @@ class HipOps:
             raise KernelError(f"the HIP kernel library could not be built or loaded: {e}") from None
         _bind(self.lib, _CORE_SIGS)
         self._attn = {}
+        self._sample_ws = {}
         self.force_linear = 0           # tests: 1 plain, 2 skinny, 3 tiled (6: its wide tile)
         self.force_plain_attention = False
 
@@ -413,6 +415,13 @@ class HipOps:
         if uniforms.dtype != torch.float32 or uniforms.numel() != logits.shape[0] or not uniforms.is_contiguous():
             raise KernelError("sample: one float32 uniform number per row")
         out = torch.empty(logits.shape[0], dtype=torch.int32, device=self.device)
-        self._call(self.lib, "tp_sample", logits.data_ptr(), logits.shape[0], logits.shape[1], float(temperature),
-                   int(top_k), float(top_p), uniforms.data_ptr(), out.data_ptr(), self._stream())
+        # the candidate filter's workspace starts zeroed and every call leaves it zeroed again: kept between calls
+        shape = tuple(logits.shape)
+        if shape not in self._sample_ws:
+            nbytes = self.lib.tp_sample_workspace_bytes(shape[0], shape[1])
+            self._sample_ws[shape] = torch.zeros(nbytes, dtype=torch.uint8, device=self.device) if nbytes else None
+        ws = self._sample_ws[shape]
+        self._call(self.lib, "tp_sample", logits.data_ptr(), shape[0], shape[1], float(temperature),
+                   int(top_k), float(top_p), uniforms.data_ptr(), out.data_ptr(), ws.data_ptr() if ws is not None else None,
+                   self._stream())
         return out
