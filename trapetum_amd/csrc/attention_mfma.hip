@@ -64,8 +64,17 @@ struct PrefillArgs {
 
 namespace {
 constexpr int BKV = 32;
-constexpr int KLD = HDP + 8;                    // LDS row strides in elements: 16 bytes of padding spread the banks
-constexpr int VLD = BKV + 8;
+// LDS layouts of a key tile, both in rows of 128 bytes whose 16-byte chunks sit at chunk ^ (row & 7): the 16 rows
+// x 4 chunks that a fragment read touches then spread over the banks (padded rows lost 43 % of the LDS cycles to
+// conflicts).  K: sub-tiles of 64 head elements, a row per key.  V transposed: two head elements per row, 32 key
+// slots (64 bytes) each.
+constexpr int KSUB = (HDP + 63) / 64;
+__device__ __forceinline__ int k_at(int key, int d) {
+    return (d >> 6) * (BKV * 64) + key * 64 + ((((d & 63) >> 3) ^ (key & 7)) << 3) + (d & 7);
+}
+__device__ __forceinline__ int v_at(int d, int slot_chunk) {
+    return (d >> 1) * 64 + (((((d & 1) << 2) | slot_chunk) ^ ((d >> 1) & 7)) << 3);
+}
 }
 
 // V of the step, transposed once per layer so that the attention blocks copy it into LDS as it lies:
@@ -109,7 +118,7 @@ namespace {
 constexpr int PTH = 512;                                         // threads of a prefill block
 constexpr int PGROUPS = 2;
 constexpr int PKEYS = PGROUPS * BKV;                             // keys staged per round
-constexpr int KS_ELEMS = BKV * KLD, VT_ELEMS = HD * VLD;         // one tile's K and V^T in LDS
+constexpr int KS_ELEMS = KSUB * BKV * 64, VT_ELEMS = HD * BKV;    // one tile's K and V^T in LDS
 constexpr int MERGE_LANE = HD / 4 + 4;                           // group 1's state per lane: its output tiles, max, sum (16-byte rows)
 constexpr int MERGE_FLOATS = 4 * 64 * MERGE_LANE;
 constexpr size_t PREFILL_LDS_TILES = (size_t)PGROUPS * (KS_ELEMS + VT_ELEMS) * sizeof(bf16_t);
@@ -119,8 +128,8 @@ constexpr size_t PREFILL_LDS = PREFILL_LDS_TILES > MERGE_FLOATS * sizeof(float) 
 __global__ void __launch_bounds__(PTH)
 attn_prefill_k(PrefillArgs a) {
     extern __shared__ __attribute__((aligned(16))) unsigned char prefill_lds[];
-    bf16_t* Ks_all = reinterpret_cast<bf16_t*>(prefill_lds);                       // [group][BKV][KLD]
-    bf16_t* Vt_all = Ks_all + PGROUPS * KS_ELEMS;                                  // [group][HD][VLD]
+    bf16_t* Ks_all = reinterpret_cast<bf16_t*>(prefill_lds);                       // [group] tiles laid out by k_at
+    bf16_t* Vt_all = Ks_all + PGROUPS * KS_ELEMS;                                  // [group] tiles laid out by v_at
     const int tid = threadIdx.x, grp = tid >> 8, wave = (tid >> 6) & 3, lane = tid & 63, c = lane & 15, g = lane >> 4;
     const bf16_t* Ks = Ks_all + grp * KS_ELEMS;
     const bf16_t* Vt = Vt_all + grp * VT_ELEMS;
@@ -141,7 +150,7 @@ attn_prefill_k(PrefillArgs a) {
     if (HDP > HD)                                   // the padding columns of K stay zero for the whole kernel
         for (int i = tid; i < PKEYS * (HDP - HD); i += PTH) {
             const int key = i / (HDP - HD);
-            Ks_all[(key / BKV) * KS_ELEMS + (key % BKV) * KLD + HD + i % (HDP - HD)] = 0;
+            Ks_all[(key / BKV) * KS_ELEMS + k_at(key % BKV, HD + i % (HDP - HD))] = 0;
         }
 
     f32x4 o[HD / 16];
@@ -183,14 +192,14 @@ attn_prefill_k(PrefillArgs a) {
             const int i = tid + t * PTH;
             const int key = i / NCH;
             if (i < PKEYS * NCH)
-                *reinterpret_cast<uint4*>(Ks_all + (key / BKV) * KS_ELEMS + (key % BKV) * KLD + (i % NCH) * 8) = fk[t].u;
+                *reinterpret_cast<uint4*>(Ks_all + (key / BKV) * KS_ELEMS + k_at(key % BKV, (i % NCH) * 8)) = fk[t].u;
         }
 #pragma unroll
         for (int t = 0; t < VTASKS; t++) {
             const int i = tid + t * PTH;
             const int d = i >> 3, part = i & 7;                      // slots part*8 .. +7 of the round: tile part / 4
             if (i < HD * 8)
-                *reinterpret_cast<uint4*>(Vt_all + (part >> 2) * VT_ELEMS + d * VLD + (part & 3) * 8) = fv[t].u;
+                *reinterpret_cast<uint4*>(Vt_all + (part >> 2) * VT_ELEMS + v_at(d, part & 3)) = fv[t].u;
         }
     };
     fetch(k_lo);
@@ -210,7 +219,7 @@ attn_prefill_k(PrefillArgs a) {
 #pragma unroll
             for (int ks = 0; ks < KSTEPS; ks++) {
                 Frag kf;
-                kf.u = *reinterpret_cast<const uint4*>(Ks + (j * 16 + c) * KLD + ks * 32 + g * 8);
+                kf.u = *reinterpret_cast<const uint4*>(Ks + k_at(j * 16 + c, ks * 32 + g * 8));
                 s[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qf[ks], s[j], 0, 0, 0);
             }
         }
@@ -257,7 +266,7 @@ attn_prefill_k(PrefillArgs a) {
 #pragma unroll
         for (int dt = 0; dt < HD / 16; dt++) {
             Frag vf;
-            vf.u = *reinterpret_cast<const uint4*>(Vt + (dt * 16 + c) * VLD + g * 8);
+            vf.u = *reinterpret_cast<const uint4*>(Vt + v_at(dt * 16 + c, g));
             if (rescale) o[dt] = o[dt] * alpha;
             o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf.v, o[dt], 0, 0, 0);
         }
