@@ -4,8 +4,9 @@ A decode step is some three hundred small launches; replaying them from a graph 
 the step (the reference reports the same lever for its own loop: runtime/README.md:49-58, and wraps capture
 and replay in `Graph`, runtime/src/lib.rs:1211-1236).  What changes from step to step (slots, positions,
 lengths, page tables, tokens) lives at fixed device addresses that are refilled before each replay; page
-tables have the cache's widest width, and launch geometry that depends on lengths is sized for the cache's
-context.  No memset node is recorded: buffers are filled by copies and kernels.
+tables have the cache's widest width, and launch geometry that depends on lengths (the slices of the decode
+attention) is sized for the graph's bound on the lengths.  No memset node is recorded: buffers are filled by
+copies and kernels.
 """
 import torch
 
