@@ -10,7 +10,8 @@ TOL = {"float32": 1e-5, "bfloat16": 2e-2}
 
 
 @pytest.fixture(scope="module", params=[("A", "float32"), ("A", "bfloat16"), ("B", "float32"), ("B", "bfloat16"),
-                                        ("C", "float32"), ("C", "bfloat16")], ids=lambda p: f"{p[0]}-{p[1]}")
+                                        ("C", "float32"), ("C", "bfloat16"), ("D", "float32"), ("D", "bfloat16")],
+                ids=lambda p: f"{p[0]}-{p[1]}")
 def setup(request, tmp_path_factory):
     from .gpu_engine import load_gpu_model
     which, dtype = request.param

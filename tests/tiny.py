@@ -31,7 +31,16 @@ TINY_C = dict(
     hidden_activation="gelu_pytorch_tanh", eos_token_id=7)
 TINY_C_INIT = dict(seed=5, sigma=0.08, sigma_norm=0.3)
 
-CONFIGS = {"A": (TINY_A, TINY_A_INIT), "B": (TINY_B, TINY_B_INIT), "C": (TINY_C, TINY_C_INIT)}
+# sizes that the matrix-core kernels do not take (a width that is no multiple of 8, a head size that is no multiple
+# of 16): the plain kernels must carry the whole model, in both precisions
+TINY_D = dict(
+    num_hidden_layers=2, hidden_size=100, num_attention_heads=5, num_key_value_heads=5, head_dim=24,
+    intermediate_size=52, vocab_size=101, rms_norm_eps=1e-6, rope_theta=100.0, sliding_window=7,
+    query_pre_attn_scalar=24, attn_logit_softcapping=30.0, final_logit_softcapping=None,
+    hidden_activation="gelu_pytorch_tanh", eos_token_id=3)
+TINY_D_INIT = dict(seed=6, sigma=0.06, sigma_norm=0.2)
+
+CONFIGS = {"A": (TINY_A, TINY_A_INIT), "B": (TINY_B, TINY_B_INIT), "C": (TINY_C, TINY_C_INIT), "D": (TINY_D, TINY_D_INIT)}
 
 
 def make_folder(tmp_path, which):
