@@ -1,5 +1,6 @@
-"""A toy mixer with a state of its own, another position table and a schedule that runs a layer twice and shares
-a cache: registered, built and stepped without a change to the framework (host logic, CPU)."""
+"""A toy mixer with a state of its own, another position table, a feed-forward with a router over experts and a
+schedule that runs a layer twice and shares a cache: registered, built and stepped without a change to the framework
+(host logic, CPU)."""
 import pytest
 import torch
 

@@ -1,5 +1,6 @@
 """The toy architecture of tests/toy_parts.py on the GPU: a mixer with a state of its own (defined in the test),
-another position table, a layer that runs twice and a run that reads another run's cache."""
+another position table, a feed-forward with a router over experts, a layer that runs twice and a run that reads
+another run's cache."""
 import pytest
 import torch
 

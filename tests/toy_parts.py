@@ -1,6 +1,7 @@
 """Toy parts defined by the tests, registered from outside the framework: a mixer with a state of fixed size
-per sequence, another position table, and an architecture that mixes them with the built-in parts.  They are
-no model of anyone's; they show that the framework's files need no change for a new part."""
+per sequence, another position table, a feed-forward with a router over experts, and an architecture that mixes
+them with the built-in parts.  They are no model of anyone's; they show that the framework's files need no change
+for a new part."""
 import dataclasses
 import math
 
@@ -9,8 +10,8 @@ import torch
 from trapetum_amd.cache import StateSpec
 from trapetum_amd.config.base import ModelConfig, key
 from trapetum_amd.models.spec import LayerSpec, ModelSpec, ScheduleEntry, TensorSpec
-from trapetum_amd.parts import Mixer, Position
-from trapetum_amd.registry import register_architecture, register_part
+from trapetum_amd.parts import FeedForward, Mixer, Position
+from trapetum_amd.registry import build_part, register_architecture, register_part
 
 
 class EmaMixer(Mixer):
@@ -44,6 +45,37 @@ class EmaMixer(Mixer):
         return ctx.ops.linear(out.to(ctx.dtype), self.w, ctx.dtype)
 
 
+class SoftRoutedMLP(FeedForward):
+    """A router over experts, each a built-in gated feed-forward: out = sum_e softmax(router(x))_e * expert_e(x).
+    Every expert runs on every row (a soft mixture), so the result is continuous in x."""
+
+    def __init__(self, hidden_size, intermediate_size, n_experts):
+        self.hidden_size, self.n_experts = hidden_size, n_experts
+        self.experts = [build_part("feed_forward", ("gated_mlp", {"hidden_size": hidden_size, "intermediate_size": intermediate_size,
+                                                                   "activation": "gelu_tanh"})) for _ in range(n_experts)]
+
+    def tensor_specs(self):
+        specs = {"router.weight": TensorSpec((self.n_experts, self.hidden_size))}
+        for e, part in enumerate(self.experts):
+            specs.update({f"experts.{e}.{name}": spec for name, spec in part.tensor_specs().items()})
+        return specs
+
+    def bind(self, tensors, rt):
+        self.rt = rt
+        self.w_router = rt.matrix(tensors["router.weight"])
+        for e, part in enumerate(self.experts):
+            head = f"experts.{e}."
+            part.bind({n[len(head):]: t for n, t in tensors.items() if n.startswith(head)}, rt)
+
+    def forward(self, ctx, x):
+        weights = torch.softmax(ctx.ops.linear(x, self.w_router, torch.float32), dim=-1)      # router logits in fp32
+        out = None
+        for e, part in enumerate(self.experts):
+            y = ctx.ops.rows(part.forward(ctx, x), torch.float32).float() * weights[:, e:e + 1]
+            out = y if out is None else out + y
+        return out.to(ctx.dtype)
+
+
 class SquaredPosition(Position):
     """Rotary frequencies d -> 1 / (1 + d)^2 over part of the head: another table through the same interface."""
 
@@ -67,6 +99,7 @@ class ToyConfig(ModelConfig):
     eps: float = key("eps", "float")
     decay: float = key("decay", "float")
     rotary: int = key("rotary", "int")
+    experts: int = key("experts", "int")
 
 
 def toy_spec(c):
@@ -80,7 +113,10 @@ def toy_spec(c):
             mixer = ("attention", {"hidden_size": c.width, "num_heads": c.heads, "num_kv_heads": c.heads,
                                    "head_dim": c.head_size, "query_scale": 1.0 / math.sqrt(c.head_size),
                                    "position": ("toy_squared", {"rotary_dim": c.rotary})})
-        ff = ("gated_mlp", {"hidden_size": c.width, "intermediate_size": c.ff_width, "activation": "gelu_tanh"})
+        if l % 2 == 0:
+            ff = ("gated_mlp", {"hidden_size": c.width, "intermediate_size": c.ff_width, "activation": "gelu_tanh"})
+        else:
+            ff = ("toy_soft_routed", {"hidden_size": c.width, "intermediate_size": c.ff_width, "n_experts": c.experts})
         layers.append(LayerSpec(block=("pre_norm", {}), mixer=mixer, feed_forward=ff, norm=norm,
                                 prefixes={"pre_mixer_norm": p + "n1.", "mixer": p + "mix.", "pre_ff_norm": p + "n2.",
                                           "feed_forward": p + "ff."}))
@@ -97,10 +133,11 @@ def toy_spec(c):
 def register():
     register_part("mixer", "toy_ema", EmaMixer)
     register_part("position", "toy_squared", SquaredPosition)
+    register_part("feed_forward", "toy_soft_routed", SoftRoutedMLP)
     register_architecture(ToyConfig.architecture, ToyConfig, toy_spec)
 
 
-TOY = dict(n_layers=2, width=48, heads=3, head_size=16, ff_width=80, vocab=97, eps=1e-5, decay=0.8, rotary=8)
+TOY = dict(n_layers=2, width=48, heads=3, head_size=16, ff_width=80, vocab=97, eps=1e-5, decay=0.8, rotary=8, experts=3)
 
 
 # ---- the toy's own plain reference: whole sequences, float64, no cache ------------------------------------------------
@@ -154,5 +191,12 @@ def toy_reference(cfg, W, tokens):
             kv1 = kv1 or kv
             x = x + a
         n = norm(x, W[p + "n2.weight"])
-        x = x + (gelu(n @ W[p + "ff.gate_proj.weight"].T) * (n @ W[p + "ff.up_proj.weight"].T)) @ W[p + "ff.down_proj.weight"].T
+
+        def mlp(t, q):
+            return (gelu(t @ W[q + "gate_proj.weight"].T) * (t @ W[q + "up_proj.weight"].T)) @ W[q + "down_proj.weight"].T
+        if l == 0:
+            x = x + mlp(n, p + "ff.")
+        else:
+            mix = torch.softmax(n @ W[p + "ff.router.weight"].T, -1)
+            x = x + sum(mix[:, e:e + 1] * mlp(n, p + f"ff.experts.{e}.") for e in range(cfg["experts"]))
     return norm(x, W["out_norm.weight"]) @ W["head.weight"].T
