@@ -50,6 +50,11 @@ def plan_batch(queue, prompts, max_tokens, max_batch, free_tokens, page_size, ma
     return taken
 
 
+def _index(like, rows):
+    import torch
+    return torch.tensor(rows, dtype=torch.long, device=like.device)
+
+
 def generate(model, cache, prompts, max_tokens=256, params=None, seed=0, stop_ids=(), max_batch=64,
              on_tokens=None, with_reasons=False, decode_step=None):
     """Generate for every prompt (lists of token ids); returns the new tokens of each, in the prompts' order.
@@ -78,8 +83,22 @@ def generate(model, cache, prompts, max_tokens=256, params=None, seed=0, stop_id
             flat = [t for i in batch for t in prompts[i]]
             logits = model.step(cache, [slots[i] for i in batch], flat, counts=[len(prompts[i]) for i in batch])
             live = list(batch)
+            step = decode_step or (lambda sl, tk: model.step(cache, sl, tk))
             while live:
-                chosen = sampler.choose(logits, [state[i] for i in live])
+                requests = [state[i] for i in live]
+                ids = sampler.choose_on_device(logits, requests)
+                fetch = model.rt.download_i32(ids)
+                # The next step is enqueued before the host knows the tokens (they stay on the device), so the GPU
+                # does not wait for the host: every sequence that its length allows to go on takes part.  One that
+                # turns out to have stopped has run one step for nothing; its row is dropped below.
+                ahead = [i for i in live if len(out[i]) + 1 < max_tokens
+                         and len(prompts[i]) + len(out[i]) + 1 <= cache.max_context]
+                next_logits = None
+                if ahead:
+                    tokens = ids if len(ahead) == len(live) else ids[_index(ids, [live.index(i) for i in ahead])]
+                    next_logits = step([slots[i] for i in ahead], tokens)
+                chosen = fetch()
+                sampler.record(requests, chosen)
                 emitted, still = [], []
                 for i, tok in zip(live, chosen):
                     if tok in stop:
@@ -98,10 +117,9 @@ def generate(model, cache, prompts, max_tokens=256, params=None, seed=0, stop_id
                 if on_tokens is not None and emitted:
                     on_tokens(step_no, emitted)
                 step_no += 1
-                live = still
-                if live:
-                    step = decode_step or (lambda sl, tk: model.step(cache, sl, tk))
-                    logits = step([slots[i] for i in live], [out[i][-1] for i in live])
+                if still and len(still) != len(ahead):
+                    next_logits = next_logits[_index(next_logits, [ahead.index(i) for i in still])]
+                live, logits = still, next_logits
         finally:
             for s in slots.values():
                 cache.release(s)

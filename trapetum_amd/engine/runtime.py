@@ -43,6 +43,23 @@ class Runtime:
             self._widened[key] = (t, t.to(self.dtype))
         return self._widened[key][1]
 
+    def download_i32(self, t):
+        """Device int32 tensor -> host, asynchronously: returns a function that waits for the copy alone (not for
+        work enqueued after it) and gives the values as a list."""
+        if self.device.type != "cuda":
+            values = t.reshape(-1).tolist()
+            return lambda: values
+        n = t.numel()
+        host = torch.empty(n, dtype=torch.int32, pin_memory=True)
+        host.copy_(t.reshape(-1), non_blocking=True)
+        ev = torch.cuda.Event()
+        ev.record()
+
+        def wait():
+            ev.synchronize()
+            return host.tolist()
+        return wait
+
     def upload_i32(self, array):
         """Host int32 numpy array -> device tensor (asynchronous from pinned memory on a GPU)."""
         t = torch.from_numpy(array)

@@ -74,6 +74,12 @@ class Sampler:
     def choose(self, logits, requests):
         """logits fp32 [n, vocab] on the device (changed in place by a penalty); one RequestSampling per row.
         Returns the chosen ids as a list, after which each request has seen its token."""
+        out = self.rt.download_i32(self.choose_on_device(logits, requests))()
+        self.record(requests, out)
+        return out
+
+    def choose_on_device(self, logits, requests):
+        """The choice as an int32 tensor on the device, nothing waited for; `record` the ids once they are known."""
         p = self.params
         ops = self.rt.ops
         if p.repetition_penalty > 1.0:
@@ -82,12 +88,12 @@ class Sampler:
                 recent[i, :len(r.recent)] = list(r.recent)
             ops.apply_repetition_penalty(logits, self.rt.upload_i32(recent), p.repetition_penalty)
         if p.temperature <= 0:
-            ids = ops.argmax(logits)
-        else:
-            u = np.asarray([r.next_uniform() for r in requests], dtype=np.float32)
-            uniforms = self.rt.upload_i32(u.view(np.int32)).view(torch.float32)
-            ids = ops.sample(logits, p.temperature, p.top_k, p.top_p, uniforms)
-        out = [int(t) for t in ids.tolist()]
-        for r, t in zip(requests, out):
-            r.saw(t)
-        return out
+            return ops.argmax(logits)
+        u = np.asarray([r.next_uniform() for r in requests], dtype=np.float32)
+        uniforms = self.rt.upload_i32(u.view(np.int32)).view(torch.float32)
+        return ops.sample(logits, p.temperature, p.top_k, p.top_p, uniforms)
+
+    @staticmethod
+    def record(requests, ids):
+        for r, t in zip(requests, ids):
+            r.saw(int(t))
