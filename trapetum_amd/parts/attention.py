@@ -10,7 +10,10 @@ reference fixes the scale to rsqrt(head_dim) (cu:249) and has no window
 t <= p, and with a window W only those with p - t < W.
 
 The three projections are one product over the concatenated weight.  A run that
-reads another run's cache projects and rotates its queries only.
+reads another run's cache projects and rotates its queries only.  In a decode step
+rotation, cache write and attention are one kernel launch where the kernel library
+has one for the geometry (`ops.fuses_decode_step`); the order of the arithmetic is
+the same.
 """
 from ..cache.store import KVSpec
 from ..models.spec import TensorSpec
