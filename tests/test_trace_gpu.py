@@ -34,7 +34,7 @@ def replay(folder, dtype, steps, out_dir, max_tokens):
     return out
 
 
-@pytest.mark.parametrize("which", ["A", "B"])
+@pytest.mark.parametrize("which", ["A", "B", "D"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_replay_schedules_agree_with_plain(which, dtype, tmp_path):
     folder = make_folder(tmp_path, which)
