@@ -136,6 +136,9 @@ struct Tile { int tm, tn; };
 static Tile pick_tile(const GemmArgs& a) {
     if (a.algo == 6) return {4, 8};
     if (a.M <= 64 && !(a.M > 32 && a.N >= 32768)) return {2, 2};    // the logits of 64 rows: 250 us with 128 x 128, 275 with 64 x 64
+    // up to 256 rows of a narrow product: 128 x 128 tiles would leave most CUs idle (down at 128 rows: 44 us
+    // on 72 blocks, against 15 us at 64 rows on 576 blocks of 64 x 64)
+    if (a.M <= 256 && (long)tp_cdiv(a.M, 128) * tp_cdiv(a.N, 128) < 256) return {2, 2};    // (at 512 rows 128 x 128 wins again)
     if ((long)tp_cdiv(a.M, 128) * tp_cdiv(a.N, 256) >= 2048) return {4, 8};
     return {4, 4};
 }
