@@ -621,6 +621,12 @@ attn_decode_combine_k(const float* __restrict__ ws_o, const float* __restrict__ 
     __shared__ float w_lds[128];
     const size_t at = (size_t)blockIdx.x * nsplit;               // blockIdx.x = sequence * heads + head
     const int tid = threadIdx.x;
+    // the first 16 slices' sums are asked for before the weights are known: both come from memory at the same time
+    constexpr int FIRST = 16;
+    const int d = tid < HD ? tid : HD - 1;                       // the block has max(HD, 64) threads
+    float o0[FIRST];
+#pragma unroll
+    for (int j = 0; j < FIRST; j++) o0[j] = ws_o[(at + (j < nsplit ? j : nsplit - 1)) * HD + d];
     if (tid < 64) {
         const int s0 = tid < nsplit ? tid : nsplit - 1, s1 = tid + 64 < nsplit ? tid + 64 : nsplit - 1;
         const float2 ml0 = *reinterpret_cast<const float2*>(ws_ml + (at + s0) * 2);
@@ -643,21 +649,24 @@ attn_decode_combine_k(const float* __restrict__ ws_o, const float* __restrict__ 
         w_lds[tid + 64] = w1 / den;
     }
     __syncthreads();
-    for (int d = tid; d < HD; d += blockDim.x) {
-        float num = 0.f;
-        for (int s0 = 0; s0 < nsplit; s0 += 8) {
-            float o[8], w[8];
+    float num = 0.f;
 #pragma unroll
-            for (int j = 0; j < 8; j++) {
-                const int s = s0 + j < nsplit ? s0 + j : nsplit - 1;
-                o[j] = ws_o[(at + s) * HD + d];
-                w[j] = s0 + j < nsplit ? w_lds[s] : 0.f;
-            }
-#pragma unroll
-            for (int j = 0; j < 8; j++) num += w[j] == 0.f ? 0.f : w[j] * o[j];
-        }
-        out[(size_t)blockIdx.x * HD + d] = f32_to_bf16(num);
+    for (int j = 0; j < FIRST; j++) {
+        const float w = j < nsplit ? w_lds[j] : 0.f;
+        num += w == 0.f ? 0.f : w * o0[j];
     }
+    for (int s0 = FIRST; s0 < nsplit; s0 += 8) {
+        float o[8], w[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const int s = s0 + j < nsplit ? s0 + j : nsplit - 1;
+            o[j] = ws_o[(at + s) * HD + d];
+            w[j] = s0 + j < nsplit ? w_lds[s] : 0.f;
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j++) num += w[j] == 0.f ? 0.f : w[j] * o[j];
+    }
+    if (tid < HD) out[(size_t)blockIdx.x * HD + tid] = f32_to_bf16(num);
 }
 
 extern "C" long tp_attn_decode_workspace_floats(int n_seq, int H, int nsplit) {
