@@ -16,6 +16,9 @@ SIZES = {
     "2b": dict(num_hidden_layers=2, hidden_size=2304, num_attention_heads=8, num_key_value_heads=4, head_dim=256,
                intermediate_size=9216, vocab_size=25601, rms_norm_eps=1e-6, rope_theta=10000.0, sliding_window=96,
                query_pre_attn_scalar=256, attn_logit_softcapping=50.0, final_logit_softcapping=30.0),
+    "9b": dict(num_hidden_layers=2, hidden_size=3584, num_attention_heads=16, num_key_value_heads=8, head_dim=256,
+               intermediate_size=14336, vocab_size=32003, rms_norm_eps=1e-6, rope_theta=10000.0, sliding_window=128,
+               query_pre_attn_scalar=256, attn_logit_softcapping=50.0, final_logit_softcapping=30.0),
     "27b-heads": dict(num_hidden_layers=2, hidden_size=1152, num_attention_heads=32, num_key_value_heads=16, head_dim=128,
                       intermediate_size=4608, vocab_size=10007, rms_norm_eps=1e-6, rope_theta=10000.0, sliding_window=80,
                       query_pre_attn_scalar=144, attn_logit_softcapping=50.0, final_logit_softcapping=30.0),
