@@ -6,42 +6,47 @@
 // (runtime/cuda/codebook_gemv.cu:86-114); its only dense one is gemv_fp16_warp_k (cu:496-517).
 #include "gemm.h"
 
-template <typename TI, typename TO>
+// A block of 16 x 16 threads owns a tile of 16 R x 16 R outputs, R x R per thread, and walks K in steps of BK
+// through LDS.  Every output is one chain acc = fma(x, w, acc) over k = 0, 1, 2, ...: the same bits for every R,
+// BK and batch.  R = 4 for many rows; R = 1 (sixteen times the blocks, whole 256-byte pieces of a row per load)
+// for the few rows of a decode step, where a narrow product would otherwise run on a few dozen blocks.
+template <typename TI, typename TO, int R, int BK>
 __global__ void __launch_bounds__(256)
 gemm_simple_k(const TI* __restrict__ X, const TI* __restrict__ W, TO* __restrict__ Y, int M, int N, int K, float cap) {
-    __shared__ float xs[16][65];
-    __shared__ float ws[16][65];
+    constexpr int T = 16 * R;
+    __shared__ float xs[BK][T + 1];
+    __shared__ float ws[BK][T + 1];
     const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
-    const int m0 = blockIdx.y * 64, n0 = blockIdx.x * 64;
-    float acc[4][4] = {};
-    for (int k0 = 0; k0 < K; k0 += 16) {
+    const int m0 = blockIdx.y * T, n0 = blockIdx.x * T;
+    float acc[R][R] = {};
+    for (int k0 = 0; k0 < K; k0 += BK) {
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int idx = tid + i * 256, r = idx >> 4, kk = idx & 15;
+        for (int i = 0; i < T * BK / 256; i++) {
+            const int idx = tid + i * 256, r = idx / BK, kk = idx % BK;
             const int k = k0 + kk;
             xs[kk][r] = (m0 + r < M && k < K) ? ld_f32(X + (size_t)(m0 + r) * K + k) : 0.f;
             ws[kk][r] = (n0 + r < N && k < K) ? ld_f32(W + (size_t)(n0 + r) * K + k) : 0.f;
         }
         __syncthreads();
+#pragma unroll 16
+        for (int kk = 0; kk < BK; kk++) {
+            float a[R], b[R];
 #pragma unroll
-        for (int kk = 0; kk < 16; kk++) {
-            float a[4], b[4];
+            for (int i = 0; i < R; i++) { a[i] = xs[kk][ty * R + i]; b[i] = ws[kk][tx * R + i]; }
 #pragma unroll
-            for (int i = 0; i < 4; i++) { a[i] = xs[kk][ty * 4 + i]; b[i] = ws[kk][tx * 4 + i]; }
+            for (int i = 0; i < R; i++)
 #pragma unroll
-            for (int i = 0; i < 4; i++)
-#pragma unroll
-                for (int j = 0; j < 4; j++) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+                for (int j = 0; j < R; j++) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
         }
         __syncthreads();
     }
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const int m = m0 + ty * 4 + i;
+    for (int i = 0; i < R; i++) {
+        const int m = m0 + ty * R + i;
         if (m >= M) continue;
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const int n = n0 + tx * 4 + j;
+        for (int j = 0; j < R; j++) {
+            const int n = n0 + tx * R + j;
             if (n >= N) continue;
             float v = acc[i][j];
             if (cap > 0.f) v = softcap_f(v, cap);
@@ -54,11 +59,19 @@ extern "C" int tp_gated_act(const float* y, void* out, int dtype, int M, int I, 
 
 template <typename TI>
 static int simple_typed(const GemmArgs& a, void* y, int out_dtype, float cap) {
+    if (a.M <= 16) {
+        dim3 grid(tp_cdiv(a.N, 16), 1);
+        if (out_dtype == TP_F32)
+            gemm_simple_k<TI, float, 1, 64><<<grid, 256, 0, a.stream>>>((const TI*)a.x, (const TI*)a.w, (float*)y, a.M, a.N, a.K, cap);
+        else
+            gemm_simple_k<TI, bf16_t, 1, 64><<<grid, 256, 0, a.stream>>>((const TI*)a.x, (const TI*)a.w, (bf16_t*)y, a.M, a.N, a.K, cap);
+        return tp_check_launch("linear (plain kernel, few rows)");
+    }
     dim3 grid(tp_cdiv(a.N, 64), tp_cdiv(a.M, 64));
     if (out_dtype == TP_F32)
-        gemm_simple_k<TI, float><<<grid, 256, 0, a.stream>>>((const TI*)a.x, (const TI*)a.w, (float*)y, a.M, a.N, a.K, cap);
+        gemm_simple_k<TI, float, 4, 16><<<grid, 256, 0, a.stream>>>((const TI*)a.x, (const TI*)a.w, (float*)y, a.M, a.N, a.K, cap);
     else
-        gemm_simple_k<TI, bf16_t><<<grid, 256, 0, a.stream>>>((const TI*)a.x, (const TI*)a.w, (bf16_t*)y, a.M, a.N, a.K, cap);
+        gemm_simple_k<TI, bf16_t, 4, 16><<<grid, 256, 0, a.stream>>>((const TI*)a.x, (const TI*)a.w, (bf16_t*)y, a.M, a.N, a.K, cap);
     return tp_check_launch("linear (plain kernel)");
 }
 
