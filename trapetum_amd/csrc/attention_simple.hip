@@ -38,7 +38,10 @@ attn_simple_k(AttnSimpleArgs a) {
         o[j] = 0.f;
     }
     float m = -INFINITY, l = 0.f;
-    for (int t = lo; t <= p; t++) {
+    // a key's row and value row are fetched while the two keys before it are worked on (the arithmetic per key, and
+    // its order, stay as they are: the loop would otherwise pay a trip to memory, or two through the page table, per key)
+    auto fetch = [&](int t, float (&kk)[4], float (&vv)[4]) {
+        t = t < p ? t : p;                               // past the last key: a row that exists, never used
         const T *kp, *vp;
         if (a.paged) {
             const int row = a.rows_cap > 0 ? t % a.rows_cap : t;
@@ -51,14 +54,19 @@ attn_simple_k(AttnSimpleArgs a) {
             kp = (const T*)a.k + row * a.k_stride + (size_t)g * a.hd;
             vp = (const T*)a.v + row * a.v_stride + (size_t)g * a.hd;
         }
-        float part = 0.f, vv[4];
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             const int d = lane + 64 * j;
-            const bool ok = d < a.hd;
-            part = fmaf(qv[j], ok ? ld_f32(kp + d) : 0.f, part);
-            vv[j] = ok ? ld_f32(vp + d) : 0.f;
+            const int dc = d < a.hd ? d : 0;
+            const float kx = ld_f32(kp + dc), vx = ld_f32(vp + dc);
+            kk[j] = d < a.hd ? kx : 0.f;
+            vv[j] = d < a.hd ? vx : 0.f;
         }
+    };
+    auto use = [&](const float (&kk)[4], const float (&vv)[4]) {
+        float part = 0.f;
+#pragma unroll
+        for (int j = 0; j < 4; j++) part = fmaf(qv[j], kk[j], part);
         float s = wave_sum(part) * a.scale;
         if (a.cap > 0.f) s = softcap_f(s, a.cap);
         const float m_new = fmaxf(m, s);
@@ -67,6 +75,19 @@ attn_simple_k(AttnSimpleArgs a) {
 #pragma unroll
         for (int j = 0; j < 4; j++) o[j] = o[j] * alpha + pr * vv[j];
         m = m_new;
+    };
+    float k0[4], v0[4], k1[4], v1[4], k2[4], v2[4];
+    fetch(lo, k0, v0);
+    fetch(lo + 1, k1, v1);
+    for (int t = lo; t <= p; t += 3) {
+        fetch(t + 2, k2, v2);
+        use(k0, v0);
+        if (t + 1 > p) break;
+        fetch(t + 3, k0, v0);
+        use(k1, v1);
+        if (t + 2 > p) break;
+        fetch(t + 4, k1, v1);
+        use(k2, v2);
     }
     T* out = (T*)a.out + ((size_t)r * a.H + h) * a.hd;
     const float inv = 1.f / l;
