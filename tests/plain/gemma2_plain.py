@@ -225,12 +225,18 @@ def repetition_penalty(logits, recent, penalty):
 def sample(logits, temperature, top_p, top_k, u):
     """Greedy for temperature <= 0; else the top_k largest (ties: smaller id first),
     softmax((z - max) / T), the shortest prefix whose mass reaches top_p, and a walk
-    with r = u * kept mass.  runtime/src/bin/serve.rs:41-72 (top_k is 256 there)."""
+    with r = u * kept mass.  runtime/src/bin/serve.rs:41-72 (top_k is 256 there).
+    top_k 0 (not in the reference): the whole vocabulary in id order, no nucleus."""
     z = [float(v) for v in logits]
     if temperature <= 0:
         return argmax(z)
-    idx = sorted(range(len(z)), key=lambda i: (-z[i], i))[:top_k if top_k > 0 else len(z)]
-    mx = z[idx[0]]
+    if top_k > 0:
+        idx = sorted(range(len(z)), key=lambda i: (-z[i], i))[:top_k]
+        mx = z[idx[0]]
+    else:
+        assert top_p >= 1
+        idx = list(range(len(z)))
+        mx = max(z)
     probs = [math.exp((z[i] - mx) / temperature) for i in idx]
     total = sum(probs)
     probs = [p / total for p in probs]

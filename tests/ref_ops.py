@@ -193,9 +193,12 @@ def sample(logits, temperature, top_k, top_p, uniforms):
     for b in range(logits.shape[0]):
         z = logits[b].double()
         k = min(top_k, z.numel()) if top_k > 0 else z.numel()
-        order = sorted(range(z.numel()), key=lambda i: (-float(z[i]), i))[:k]
+        if top_k > 0:
+            order = sorted(range(z.numel()), key=lambda i: (-float(z[i]), i))[:k]
+        else:
+            order = list(range(z.numel()))            # the whole vocabulary, in id order, no nucleus
         zs = torch.tensor([float(z[i]) for i in order], dtype=torch.float64)
-        p = torch.exp((zs - zs[0]) / temperature)
+        p = torch.exp((zs - zs.max()) / temperature)
         p = p / p.sum()
         cum = torch.cumsum(p, 0)
         keep = k

@@ -31,25 +31,27 @@ def test_greedy_generation_equals_plain_loop(folders, use_graph):
     assert got[1].reason == "stop" and len(got[1].tokens) == 3
 
 
-def test_sampled_generation_equals_plain_sampler(folders):
-    """Temperature 0.7, seed 7 (tiny B): with the same uniform numbers the plain sampler picks the same tokens."""
+@pytest.mark.parametrize("top_p,top_k", [(0.9, 50), (1.0, 0)])
+def test_sampled_generation_equals_plain_sampler(folders, top_p, top_k):
+    """Temperature 0.7, seed 7 (tiny B): with the same uniform numbers the plain sampler picks the same tokens, from a
+    nucleus of the 50 largest and from the whole vocabulary."""
     from trapetum_amd import load_model
     from trapetum_amd.sampling import initial_state
     pcfg, pw = plain.read_folder(folders["B"])
     engine = load_model(folders["B"], dtype="float32", max_tokens_in_cache=2048)
     prompts = [random_tokens(n, pcfg["vocab_size"], 80 + n) for n in (1, 9, 23, 40)]
-    got = engine.generate(prompts, max_tokens=12, temperature=0.7, top_p=0.9, top_k=50, seed=7, stop_ids=())
+    got = engine.generate(prompts, max_tokens=12, temperature=0.7, top_p=top_p, top_k=top_k, seed=7, stop_ids=())
     for i, p in enumerate(prompts):
         state, seq, out = initial_state(7, i), list(p), []
         for _ in range(12):
             state = plain.xorshift64(state)
             u = float(torch.tensor(plain.uniform_from_state(state), dtype=torch.float32))
-            tok = plain.sample(plain.forward(pcfg, pw, seq)[-1], 0.7, 0.9, 50, u)
+            tok = plain.sample(plain.forward(pcfg, pw, seq)[-1], 0.7, top_p, top_k, u)
             out.append(tok)
             seq.append(tok)
         assert got[i] == out, i
     # each request alone gives what it gave in the batch
-    alone = engine.generate([prompts[2]], max_tokens=12, temperature=0.7, top_p=0.9, top_k=50, seed=7, stop_ids=())
+    alone = engine.generate([prompts[2]], max_tokens=12, temperature=0.7, top_p=top_p, top_k=top_k, seed=7, stop_ids=())
     assert alone[0] != [] and len(alone[0]) == 12
 
 

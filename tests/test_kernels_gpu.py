@@ -346,7 +346,8 @@ def test_argmax_ties_and_nan(ops):
 
 # ---- token choice ----------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("vocab,temperature,top_k,top_p", [(256, 0.7, 256, 0.95), (7001, 1.0, 40, 1.0), (7001, 0.3, 1000, 0.5),
-                                                           (256000, 0.9, 256, 0.95), (513, 1.5, 1, 1.0), (513, 0.8, 600, 0.99)])
+                                                           (256000, 0.9, 256, 0.95), (513, 1.5, 1, 1.0), (513, 0.8, 600, 0.99), (513, 0.8, 0, 1.0),
+                                                           (50001, 1.2, 0, 1.0)])
 def test_sample_follows_the_plain_sampler(ops, vocab, temperature, top_k, top_p):
     """Sort by logit (ties: smaller id), keep top_k, softmax at the temperature, shortest prefix reaching top_p, walk
     with u (runtime/src/bin/serve.rs:41-72).  Ties and a dominant token are planted; where the uniform number falls
@@ -358,6 +359,8 @@ def test_sample_follows_the_plain_sampler(ops, vocab, temperature, top_k, top_p)
     u = torch.tensor([0.0, 0.5, 0.999, 0.25, 0.75, 0.9999], dtype=torch.float32)
     with pytest.raises(Exception, match="top_k"):            # the kernel sorts at most 1024 candidates and says so
         ops.sample(z.to(DEV), temperature, 2000, top_p, u.to(DEV))
+    with pytest.raises(Exception, match="nucleus"):          # the whole vocabulary (top_k 0) goes without a nucleus
+        ops.sample(z.to(DEV), temperature, 0, 0.9, u.to(DEV))
     got = ops.sample(z.to(DEV), temperature, top_k, top_p, u.to(DEV)).cpu().tolist()
     for b in range(rows):
         choices = set()

@@ -24,7 +24,7 @@ def _add_sampling(ap):
     ap.add_argument("--max-tokens", type=int, default=24, help="tokens to generate per prompt (gemma_run generates 24)")
     ap.add_argument("--temperature", type=float, default=0.0, help="0 = greedy")
     ap.add_argument("--top-p", type=float, default=0.95)
-    ap.add_argument("--top-k", type=int, default=256)
+    ap.add_argument("--top-k", type=int, default=256, help="candidates kept (the reference keeps 256); 0: the whole vocabulary, with --top-p 1")
     ap.add_argument("--repetition-penalty", type=float, default=1.0)
     ap.add_argument("--seed", type=int, default=0, help="sampling seed")
     ap.add_argument("--stop-id", type=int, action="append", default=None,

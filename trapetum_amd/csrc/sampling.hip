@@ -326,6 +326,60 @@ sample_k(const float* __restrict__ logits, int V, float temperature, int top_k, 
     }
 }
 
+// ---- temperature sampling over the whole vocabulary (top_k 0, no nucleus; the reference always keeps 256): p_i =
+// exp((z_i - max) / T), r = u * sum, the token whose cumulative mass in id order first exceeds r.  One block per
+// row; thread t owns a contiguous range of ids, so sums run over ids in order within a thread, then over the threads
+// in order. ----------------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(1024)
+sample_full_k(const float* __restrict__ logits, int V, float temperature, const float* __restrict__ uniforms,
+              int* __restrict__ out) {
+    __shared__ float part[1024];
+    __shared__ float s_total;
+    __shared__ int s_winner;
+    const float* z = logits + (size_t)blockIdx.x * V;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    float mx = -INFINITY;
+    for (int i = tid; i < V; i += 1024) { const float v = z[i]; mx = v > mx ? v : mx; }      // NaN never wins
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+    if (lane == 0) part[wave] = mx;
+    __syncthreads();
+    mx = part[0];
+    for (int w = 1; w < 16; w++) mx = fmaxf(mx, part[w]);
+    __syncthreads();
+    const int chunk = (V + 1023) / 1024, begin = tid * chunk, end = min(V, begin + chunk);
+    float mine = 0.f;
+    for (int i = begin; i < end; i++) { const float v = z[i]; mine += v == v ? expf((v - mx) / temperature) : 0.f; }
+    part[tid] = mine;
+    __syncthreads();
+    if (tid < 64) {                                  // the first wave: totals of 16 threads per lane, then over the lanes
+        float local = 0.f;
+        for (int j = 0; j < 16; j++) local += part[tid * 16 + j];
+        const float incl = wave_scan_incl(local, tid);
+        float run = incl - local;
+        for (int j = 0; j < 16; j++) { const float v = part[tid * 16 + j]; part[tid * 16 + j] = run; run += v; }   // exclusive sums
+        if (tid == 63) s_total = incl;
+    }
+    __syncthreads();
+    const float r = uniforms[blockIdx.x] * s_total;
+    const float before = part[tid];
+    // the first thread whose range reaches past r walks it; rounding may leave r past every range: the last one
+    if (tid == 0) s_winner = (V - 1) / chunk;
+    __syncthreads();
+    if (begin < end && r < before + mine) atomicMin(&s_winner, tid);
+    __syncthreads();
+    if (tid == s_winner) {
+        float run = before;
+        int pick = end - 1;
+        for (int i = begin; i < end; i++) {
+            const float v = z[i];
+            run += v == v ? expf((v - mx) / temperature) : 0.f;
+            if (r < run) { pick = i; break; }
+        }
+        out[blockIdx.x] = pick;
+    }
+}
+
 // ---- a coarse filter in front of the exact sampler, on many blocks: the sampler alone reads a row of 256,000
 // logits several times on one CU (0.4 ms).  A histogram of the top 12 bits of the value keys gives the bin that
 // holds the top_k-th largest logit; everything from that bin upwards (top_k plus that bin's other members, a few
@@ -431,10 +485,15 @@ extern "C" int tp_sample(const float* logits, int B, int V, float temperature, i
                          const float* uniforms, int* out, void* workspace, void* stream) {
     TP_REQUIRE(B > 0 && V > 0, "sample: empty shape B=%d V=%d", B, V);
     TP_REQUIRE(temperature > 0.f, "sample: temperature %g must be positive (0 means argmax)", temperature);
-    TP_REQUIRE(top_k >= 1 && top_k <= 1024, "sample: top_k %d must lie in 1..1024", top_k);
+    TP_REQUIRE(top_k >= 0 && top_k <= 1024, "sample: top_k %d must lie in 0..1024 (0: the whole vocabulary)", top_k);
     TP_REQUIRE(top_p > 0.f, "sample: top_p %g must be positive", top_p);
+    TP_REQUIRE(top_k > 0 || top_p >= 1.f, "sample: a nucleus (top_p %g) needs top_k between 1 and 1024", top_p);
     TP_REQUIRE(B <= 65535, "sample: %d rows exceed one launch", B);
     hipStream_t s = (hipStream_t)stream;
+    if (top_k == 0) {
+        sample_full_k<<<B, 1024, 0, s>>>(logits, V, temperature, uniforms, out);
+        return tp_check_launch("sample (whole vocabulary)");
+    }
     if (!workspace || tp_sample_workspace_bytes(B, V) == 0) {
         sample_k<<<B, 1024, 0, s>>>(logits, V, temperature, top_k, top_p, uniforms, out, nullptr, nullptr, nullptr, 0);
         return tp_check_launch("sample");

@@ -23,14 +23,16 @@ MAX_TOP_K = 1024
 class SamplingParams:
     temperature: float = 0.0            # 0 (or less): greedy
     top_p: float = 0.95                 # the reference's default (serve.rs:1292)
-    top_k: int = 256                    # the reference keeps the 256 largest (serve.rs:52)
+    top_k: int = 256                    # the reference keeps the 256 largest (serve.rs:52); 0: the whole vocabulary, in id order
     repetition_penalty: float = 1.0     # 1 (or less): off
 
     def validate(self):
-        if not 1 <= self.top_k <= MAX_TOP_K:
-            raise ValueError(f"top_k {self.top_k} must lie in 1..{MAX_TOP_K}")
+        if not 0 <= self.top_k <= MAX_TOP_K:
+            raise ValueError(f"top_k {self.top_k} must lie in 0..{MAX_TOP_K} (0: the whole vocabulary)")
         if not self.top_p > 0:
             raise ValueError(f"top_p {self.top_p} must be positive")
+        if self.top_k == 0 and self.top_p < 1:
+            raise ValueError(f"a nucleus (top_p {self.top_p}) needs top_k between 1 and {MAX_TOP_K}")
 
 
 def xorshift64(state):
