@@ -333,6 +333,41 @@ def test_attention_far_key_stands_out(ops):
             assert rel_l2(got, want) < 2e-2, (target, plain)
 
 
+@pytest.mark.parametrize("window,rows_cap,lens", [(4096, 4096, (5000, 4100, 4096, 9000)), (0, 0, (5000, 8191, 63, 64)),
+                                                  (1000, 1024, (1000, 1001, 3333, 2048))])
+def test_attention_decode_long_contexts(ops, window, rows_cap, lens):
+    """Thousands of keys at the 2B head size: rings that have wrapped once and twice, a window shorter than its ring,
+    lengths at and beside a page's end, pages scattered over the pool, and every way of cutting the keys into slices."""
+    H, KV, hd, page, scale, cap = 8, 4, 256, 64, 1 / 16.0, 50.0
+    g = torch.Generator().manual_seed(5)
+    n = len(lens)
+    per = [-(-(min(l, rows_cap) if rows_cap else l) // page) for l in lens]
+    n_pages = sum(per) + 3
+    kp, vp = (torch.zeros(n_pages, KV, page, hd, dtype=torch.bfloat16) for _ in range(2))
+    free = torch.randperm(n_pages, generator=g).tolist()
+    table = torch.full((n, max(per)), -1, dtype=torch.int32)
+    q = (torch.randn(n, H, hd, generator=g) * 0.5).to(torch.bfloat16)
+    ref = torch.zeros(n, H, hd)
+    for i, l in enumerate(lens):
+        table[i, :per[i]] = torch.tensor([free.pop() for _ in range(per[i])], dtype=torch.int32)
+        k = (torch.randn(l, KV, hd, generator=g) * 0.5).to(torch.bfloat16)
+        v = torch.randn(l, KV, hd, generator=g).to(torch.bfloat16)
+        kept = torch.arange(max(0, l - rows_cap) if rows_cap else 0, l)            # what the ring still holds
+        rows = kept % rows_cap if rows_cap else kept
+        pages = table[i].long()[rows // page]
+        kp[pages, :, rows % page] = k[kept]
+        vp[pages, :, rows % page] = v[kept]
+        lo = max(0, l - window) if window else 0
+        scores = torch.einsum("tgd,gqd->gqt", k[lo:].float(), q[i].float().reshape(KV, H // KV, hd)) * scale
+        weights = torch.softmax(cap * torch.tanh(scores / cap), dim=-1)
+        ref[i] = torch.einsum("gqt,tgd->gqd", weights, v[lo:].float()).reshape(H, hd)
+    for splits in (None, 1, 7, 33, 128):
+        got = ops.attention_decode(q.reshape(n, H * hd).to(DEV), H, KV, hd, torch.tensor(lens, dtype=torch.int32, device=DEV),
+                                   table.to(DEV), kp.to(DEV), vp.to(DEV), rows_cap, scale, cap, window, torch.bfloat16,
+                                   max_keys=max(lens), splits=splits)
+        assert rel_l2(got.reshape(n, H, hd), ref) < 8e-3, splits
+
+
 def test_argmax_ties_and_nan(ops):
     z = torch.full((3, 7001), -1.0)
     z[0, 100] = z[0, 7000] = 5.0               # tie: the smaller index wins (runtime/src/bin/opt_check.rs:37-65)
