@@ -223,6 +223,29 @@ def test_attention_prefill(ops, plain, dt, H, KV, hd, lens, page, window, rows_c
     assert rel_l2(got, ref) < (3e-6 if dt == "f32" else 8e-3)
 
 
+@pytest.mark.parametrize("H,KV,hd,lens,window,cap", [(64, 8, 16, (450, 130, 64), 100, 30.0), (8, 4, 256, (3300,), 0, 50.0),
+                                                    (8, 4, 256, (1000, 77), 300, 0.0)])
+def test_attention_prefill_many_tiles(ops, H, KV, hd, lens, window, cap):
+    """Steps of many and of few query tiles (the kernel cuts them into blocks of 64 and of 32 queries), against
+    dense masked attention per sequence and head."""
+    m, g, scale = sum(lens), H // KV, 1.0 / math.sqrt(hd * 0.7)
+    q, k, v = (randn(m, n * hd, dtype=torch.bfloat16, seed=40 + i) for i, n in enumerate((H, KV, KV)))
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
+    ref = torch.zeros(m, H, hd)
+    for i, n in enumerate(lens):
+        rows = slice(int(cu[i]), int(cu[i + 1]))
+        qs, ks, vs = (t.cpu().float()[rows].reshape(n, -1, hd) for t in (q, k, v))
+        pos = torch.arange(n)
+        hidden = (pos[None, :] > pos[:, None]) | ((pos[:, None] - pos[None, :] >= window) if window else False)
+        for h in range(H):
+            s = qs[:, h] @ ks[:, h // g].T * scale
+            if cap:
+                s = cap * torch.tanh(s / cap)
+            ref[rows, h] = torch.softmax(s.masked_fill(hidden, float("-inf")), dim=-1) @ vs[:, h // g]
+    got = ops.attention_prefill(q, k, v, H, KV, hd, cu.to(DEV), max(lens), scale, cap, window, torch.bfloat16)
+    assert rel_l2(got.reshape(m, H, hd), ref) < 8e-3
+
+
 @pytest.mark.parametrize("plain", [True, False])
 @pytest.mark.parametrize("dt", ["f32", "bf16"])
 @pytest.mark.parametrize("H,KV,hd,lens,page,window,rows_cap,cap", ATTN_CASES)

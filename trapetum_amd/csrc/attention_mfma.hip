@@ -52,7 +52,7 @@ __device__ __forceinline__ bf16_t bf16_bits(float f) {
 
 // =====================================================================================================
 // prefill: every sequence of the step starts at position 0; keys and values are the step's own rows.
-// Block = 64 queries of one (sequence, head); a wave owns 16 queries.  Key tiles of 32 go through LDS: K as
+// Block = 64 or 32 queries of one (sequence, head); a wave owns 16 queries.  Key tiles of 32 go through LDS: K as
 // stored (row = key), V transposed (row = head element) with the keys of a tile permuted so that a lane's 8
 // probabilities meet the 8 values of the same keys in one 16-byte LDS read.
 // =====================================================================================================
@@ -110,31 +110,41 @@ v_transpose_k(const bf16_t* __restrict__ v, long v_stride, int KV, const int* __
     }
 }
 
-// Block = 8 waves in two groups of four, 64 queries of one (sequence, head): wave w of either group owns queries
-// w*16 .. w*16+15.  Per round the block stages two key tiles (64 keys); group 0 takes the first, group 1 the
-// second, each with its own running softmax, so the chain of dependent rounds is half as long as the keys; at
-// the end group 1 hands (max, sum, unnormalised output) to group 0 through LDS.
+// Block = 8 waves in PGROUPS groups of PWAVES, PQ queries of one (sequence, head): wave w of every group owns
+// queries w*16 .. w*16+15.  Per round the block stages PGROUPS key tiles; group i takes the i-th, each group with its
+// own running softmax, so the chain of dependent rounds is 1/PGROUPS as long as the keys; at the end the other groups
+// hand (max, sum, unnormalised output) to group 0 through LDS.  A causal tile's work grows with its place in the
+// sequence, and a block occupies a CU alone: the late (long) tiles of every head carry the lowest block ids, so the
+// short ones fill in behind them, and a step of few tiles is cut into blocks of 32 queries instead of 64.
 namespace {
 constexpr int PTH = 512;                                         // threads of a prefill block
-constexpr int PGROUPS = 2;
-constexpr int PKEYS = PGROUPS * BKV;                             // keys staged per round
 constexpr int KS_ELEMS = KSUB * BKV * 64, VT_ELEMS = HD * BKV;    // one tile's K and V^T in LDS
-constexpr int MERGE_LANE = HD / 4 + 4;                           // group 1's state per lane: its output tiles, max, sum (16-byte rows)
-constexpr int MERGE_FLOATS = 4 * 64 * MERGE_LANE;
-constexpr size_t PREFILL_LDS_TILES = (size_t)PGROUPS * (KS_ELEMS + VT_ELEMS) * sizeof(bf16_t);
-constexpr size_t PREFILL_LDS = PREFILL_LDS_TILES > MERGE_FLOATS * sizeof(float) ? PREFILL_LDS_TILES : MERGE_FLOATS * sizeof(float);
+constexpr int MERGE_LANE = HD / 4 + 4;                           // a group's state per lane: its output tiles, max, sum (16-byte rows)
+template <int PQ> struct PrefillShape {                          // PQ: queries of a block
+    static constexpr int PWAVES = PQ / 16;                       // waves of a group
+    static constexpr int PGROUPS = PTH / 64 / PWAVES;
+    static constexpr int PKEYS = PGROUPS * BKV;                  // keys staged per round
+    static constexpr int MERGE_GROUP = PWAVES * 64 * MERGE_LANE;
+    static constexpr size_t TILE_BYTES = (size_t)PGROUPS * (KS_ELEMS + VT_ELEMS) * sizeof(bf16_t);
+    static constexpr size_t MERGE_BYTES = (size_t)(PGROUPS - 1) * MERGE_GROUP * sizeof(float);
+    static constexpr size_t LDS_BYTES = TILE_BYTES > MERGE_BYTES ? TILE_BYTES : MERGE_BYTES;
+    static_assert(LDS_BYTES <= 160 * 1024, "a round's tiles must fit the LDS of a CU");
+};
 }
 
+template <int PQ>
 __global__ void __launch_bounds__(PTH)
 attn_prefill_k(PrefillArgs a) {
+    using Shape = PrefillShape<PQ>;
+    constexpr int PWAVES = Shape::PWAVES, PGROUPS = Shape::PGROUPS, PKEYS = Shape::PKEYS, MERGE_GROUP = Shape::MERGE_GROUP;
     extern __shared__ __attribute__((aligned(16))) unsigned char prefill_lds[];
     bf16_t* Ks_all = reinterpret_cast<bf16_t*>(prefill_lds);                       // [group] tiles laid out by k_at
     bf16_t* Vt_all = Ks_all + PGROUPS * KS_ELEMS;                                  // [group] tiles laid out by v_at
-    const int tid = threadIdx.x, grp = tid >> 8, wave = (tid >> 6) & 3, lane = tid & 63, c = lane & 15, g = lane >> 4;
+    const int tid = threadIdx.x, grp = (tid >> 6) / PWAVES, wave = (tid >> 6) % PWAVES, lane = tid & 63, c = lane & 15, g = lane >> 4;
     const bf16_t* Ks = Ks_all + grp * KS_ELEMS;
     const bf16_t* Vt = Vt_all + grp * VT_ELEMS;
     // late query tiles see the most keys: they are given the low block ids, which start first
-    const int seq = blockIdx.z, h = blockIdx.y, q0 = (gridDim.x - 1 - blockIdx.x) * 64;
+    const int seq = blockIdx.z, h = blockIdx.x % a.H, q0 = (gridDim.x / a.H - 1 - blockIdx.x / a.H) * PQ;
     const int row0 = a.cu_rows[seq], T = a.cu_rows[seq + 1] - row0;
     if (q0 >= T) return;
     const int kvh = h / (a.H / a.KV);
@@ -161,11 +171,12 @@ attn_prefill_k(PrefillArgs a) {
 
     int k_lo = a.window > 0 ? max(0, q0 - a.window + 1) : 0;
     k_lo &= ~(BKV - 1);
-    const int k_hi = min(T, q0 + 64);
+    const int k_hi = min(T, q0 + PQ);
     // a round's rows travel global memory -> registers (one round ahead, while the round before is being used) ->
-    // LDS; K as stored, V from its transposed copy: HD rows of 64 slots (128 bytes) per round
+    // LDS; K as stored, V from its transposed copy: HD rows of PKEYS slots per round
+    constexpr int VCH = PKEYS / 8;                                  // 16-byte chunks of a head element's slots in a round
     constexpr int KTASKS = (PKEYS * NCH + PTH - 1) / PTH;           // (key, 16-byte chunk) per thread
-    constexpr int VTASKS = (HD * 8 + PTH - 1) / PTH;                // (head element, 16-byte chunk of its 64 slots)
+    constexpr int VTASKS = (HD * VCH + PTH - 1) / PTH;              // (head element, chunk of its slots)
     Frag fk[KTASKS], fv[VTASKS];
     const int vbase = vt_base_of(a.cu_rows, seq);
     auto fetch = [&](int kt) {
@@ -174,15 +185,15 @@ attn_prefill_k(PrefillArgs a) {
             const int i = tid + t * PTH;
             const int key = i / NCH, ch = i % NCH, tk = kt + key;
             fk[t].u = make_uint4(0, 0, 0, 0);
-            if (i < PKEYS * NCH && tk < T)
+            if (i < PKEYS * NCH && tk < k_hi)
                 fk[t].u = *reinterpret_cast<const uint4*>(a.k + (size_t)(row0 + tk) * a.k_stride + (size_t)kvh * HD + ch * 8);
         }
 #pragma unroll
         for (int t = 0; t < VTASKS; t++) {
             const int i = tid + t * PTH;
-            const int d = i >> 3, part = i & 7;
+            const int d = i / VCH, part = i % VCH;
             fv[t].u = make_uint4(0, 0, 0, 0);
-            if (i < HD * 8 && kt + (part >> 2) * BKV < k_hi)         // a tile past the block's last key is never used
+            if (i < HD * VCH && kt + (part >> 2) * BKV < k_hi)       // a tile past the block's last key is never used
                 fv[t].u = *reinterpret_cast<const uint4*>(a.vt + ((size_t)kvh * HD + d) * a.vt_rows + vbase + kt + part * 8);
         }
     };
@@ -197,8 +208,8 @@ attn_prefill_k(PrefillArgs a) {
 #pragma unroll
         for (int t = 0; t < VTASKS; t++) {
             const int i = tid + t * PTH;
-            const int d = i >> 3, part = i & 7;                      // slots part*8 .. +7 of the round: tile part / 4
-            if (i < HD * 8)
+            const int d = i / VCH, part = i % VCH;                   // slots part*8 .. +7 of the round: tile part / 4
+            if (i < HD * VCH)
                 *reinterpret_cast<uint4*>(Vt_all + (part >> 2) * VT_ELEMS + v_at(d, part & 3)) = fv[t].u;
         }
     };
@@ -271,30 +282,56 @@ attn_prefill_k(PrefillArgs a) {
             o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf.v, o[dt], 0, 0, 0);
         }
     }
-    // ---- group 1's state joins group 0's: both rescaled to the common maximum, group 0 first ---------------------
+    // ---- the other groups' states join group 0's, in the groups' order, all rescaled to the common maximum ---------
     __syncthreads();                                 // the tiles in LDS are done with
     float* merge = reinterpret_cast<float*>(prefill_lds) + (size_t)(wave * 64 + lane) * MERGE_LANE;
-    if (grp == 1) {
+    if (grp > 0) {
+        float* mine = merge + (size_t)(grp - 1) * MERGE_GROUP;
 #pragma unroll
-        for (int dt = 0; dt < HD / 16; dt++) *reinterpret_cast<f32x4*>(merge + dt * 4) = o[dt];
-        merge[HD / 4] = m_i;
-        merge[HD / 4 + 1] = l_i;
+        for (int dt = 0; dt < HD / 16; dt++) *reinterpret_cast<f32x4*>(mine + dt * 4) = o[dt];
+        mine[HD / 4] = m_i;
+        mine[HD / 4 + 1] = l_i;
     }
     __syncthreads();
-    if (grp == 1 || !q_ok) return;
-    const float m1 = merge[HD / 4], l1 = merge[HD / 4 + 1];
-    const float m = fmaxf(m_i, m1);
-    const float a0 = m_i == -INFINITY ? 0.f : __expf(m_i - m), a1 = m1 == -INFINITY ? 0.f : __expf(m1 - m);
-    const float inv = 1.f / (l_i * a0 + l1 * a1);
+    if (grp > 0 || !q_ok) return;
+    float m = m_i;
+#pragma unroll
+    for (int j = 0; j < PGROUPS - 1; j++) m = fmaxf(m, merge[(size_t)j * MERGE_GROUP + HD / 4]);
+    const float a0 = m_i == -INFINITY ? 0.f : __expf(m_i - m);
+    float l = l_i * a0;
+#pragma unroll
+    for (int dt = 0; dt < HD / 16; dt++) o[dt] = o[dt] * a0;
+#pragma unroll
+    for (int j = 0; j < PGROUPS - 1; j++) {
+        const float* theirs = merge + (size_t)j * MERGE_GROUP;
+        const float mj = theirs[HD / 4];
+        const float aj = mj == -INFINITY ? 0.f : __expf(mj - m);
+        l += theirs[HD / 4 + 1] * aj;
+#pragma unroll
+        for (int dt = 0; dt < HD / 16; dt++) o[dt] = o[dt] + *reinterpret_cast<const f32x4*>(theirs + dt * 4) * aj;
+    }
+    const float inv = 1.f / l;
     bf16_t* orow = a.out + ((size_t)(row0 + qpos) * a.H + h) * HD;
 #pragma unroll
     for (int dt = 0; dt < HD / 16; dt++) {
-        const f32x4 o1 = *reinterpret_cast<const f32x4*>(merge + dt * 4);
         ushort4 pk;
-        pk.x = bf16_bits((o[dt][0] * a0 + o1[0] * a1) * inv); pk.y = bf16_bits((o[dt][1] * a0 + o1[1] * a1) * inv);
-        pk.z = bf16_bits((o[dt][2] * a0 + o1[2] * a1) * inv); pk.w = bf16_bits((o[dt][3] * a0 + o1[3] * a1) * inv);
+        pk.x = bf16_bits(o[dt][0] * inv); pk.y = bf16_bits(o[dt][1] * inv);
+        pk.z = bf16_bits(o[dt][2] * inv); pk.w = bf16_bits(o[dt][3] * inv);
         *reinterpret_cast<ushort4*>(orow + dt * 16 + g * 4) = pk;
     }
+}
+
+template <int PQ>
+static int prefill_launch(const PrefillArgs& a, int max_count, int H, int n_seq, hipStream_t stream) {
+    constexpr size_t lds = PrefillShape<PQ>::LDS_BYTES;
+    static bool configured = false;                                   // more LDS than a kernel gets without asking
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute((const void*)attn_prefill_k<PQ>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return tp_fail("attention prefill: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
+        configured = true;
+    }
+    attn_prefill_k<PQ><<<dim3(tp_cdiv(max_count, PQ) * H, 1, n_seq), PTH, lds, stream>>>(a);
+    return 0;
 }
 
 // elements of the transposed copy of V the prefill kernel needs as workspace
@@ -309,7 +346,7 @@ extern "C" int tp_attn_prefill(const void* q, long q_stride, const void* k, long
     TP_REQUIRE(H % KV == 0, "attention: %d query heads are no multiple of %d kv heads", H, KV);
     TP_REQUIRE(q_stride % 8 == 0 && k_stride % 8 == 0 && v_stride % 8 == 0 && (uintptr_t)q % 16 == 0 &&
                (uintptr_t)k % 16 == 0 && (uintptr_t)v % 16 == 0, "attention prefill: rows must be 16-byte aligned");
-    TP_REQUIRE(H <= 65535 && n_seq <= 65535, "attention prefill: %d heads / %d sequences exceed one launch", H, n_seq);
+    TP_REQUIRE(n_seq <= 65535 && (long)tp_cdiv(max_count, 32) * H < (1L << 31), "attention prefill: %d heads / %d sequences exceed one launch", H, n_seq);
     TP_REQUIRE(workspace && (uintptr_t)workspace % 16 == 0, "attention prefill: needs its 16-byte aligned workspace");
     TP_REQUIRE(KV <= 65535, "attention prefill: %d kv heads exceed one launch", KV);
     const long vt_rows = (long)M + (long)BKV * n_seq + BKV;         // every sequence's region is padded to whole groups
@@ -318,14 +355,12 @@ extern "C" int tp_attn_prefill(const void* q, long q_stride, const void* k, long
     if (int rc = tp_check_launch("attention prefill (transpose of V)")) return rc;
     PrefillArgs a{(const bf16_t*)q, q_stride, (const bf16_t*)k, k_stride, (const bf16_t*)v, v_stride, H, KV, cu_rows,
                   scale, cap, window, (bf16_t*)out, (const bf16_t*)workspace, vt_rows};
-    static bool configured = false;                                   // more LDS than a kernel gets without asking
-    if (!configured) {
-        hipError_t e = hipFuncSetAttribute((const void*)attn_prefill_k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)PREFILL_LDS);
-        if (e != hipSuccess) return tp_fail("attention prefill: cannot reserve %zu bytes of LDS: %s", (size_t)PREFILL_LDS, hipGetErrorString(e));
-        configured = true;
-    }
-    dim3 grid(tp_cdiv(max_count, 64), H, n_seq);
-    attn_prefill_k<<<grid, PTH, PREFILL_LDS, (hipStream_t)stream>>>(a);
+    // 64 queries a block stage each key once per 64 queries; 32 a block make twice the blocks, for grids that would
+    // leave CUs idle behind the longest tiles (measured at 2,048 tokens: 8 heads of 256 93 against 103 us with 32
+    // queries, 32 heads of 128 186 against 116 us)
+    const bool small = (long)tp_cdiv(max_count, 64) * H * n_seq <= 384;
+    if (int rc = small ? prefill_launch<32>(a, max_count, H, n_seq, (hipStream_t)stream)
+                       : prefill_launch<64>(a, max_count, H, n_seq, (hipStream_t)stream)) return rc;
     return tp_check_launch("attention prefill");
 }
 
