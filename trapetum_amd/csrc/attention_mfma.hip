@@ -166,8 +166,12 @@ attn_prefill_k(PrefillArgs a) {
     f32x4 o[HD / 16];
 #pragma unroll
     for (int dt = 0; dt < HD / 16; dt++) o[dt] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    float m_i = -INFINITY, l_i = 0.f;
-    const float soc = a.cap > 0.f ? a.scale / a.cap : 0.f;
+    float m_i = -INFINITY, l_i = 0.f;                                // the running maximum in units of log 2
+    constexpr float LOG2E = 1.4426950408889634f;
+    const float tanh_in = a.cap > 0.f ? 2.f * LOG2E * a.scale / a.cap : 0.f, cap2 = a.cap * LOG2E, scale2 = a.scale * LOG2E;
+    // the keys a lane's query sees: seen_lo .. seen_lo + seen_span
+    const int seen_lo = a.window > 0 ? max(0, qpos - a.window + 1) : 0;
+    const unsigned seen_span = (unsigned)max(0, min(qpos, T - 1) - seen_lo);
 
     int k_lo = a.window > 0 ? max(0, q0 - a.window + 1) : 0;
     k_lo &= ~(BKV - 1);
@@ -177,24 +181,39 @@ attn_prefill_k(PrefillArgs a) {
     constexpr int VCH = PKEYS / 8;                                  // 16-byte chunks of a head element's slots in a round
     constexpr int KTASKS = (PKEYS * NCH + PTH - 1) / PTH;           // (key, 16-byte chunk) per thread
     constexpr int VTASKS = (HD * VCH + PTH - 1) / PTH;              // (head element, chunk of its slots)
-    Frag fk[KTASKS], fv[VTASKS];
-    const int vbase = vt_base_of(a.cu_rows, seq);
+    bf16x8 fk[KTASKS], fv[VTASKS];
+    // Addresses: a byte offset per thread from base pointers that are the same for the whole block and move with the
+    // round (scalar work).  A chunk the round does not need reads the round's first chunk instead, so that every load
+    // is issued without a branch and nothing is computed per round and lane but a comparison and a selection.
+    constexpr bool K_EVEN = PTH % NCH == 0;                         // then task t's key is task 0's + t * PTH / NCH
+    const char* const k_origin = reinterpret_cast<const char*>(a.k + (size_t)row0 * a.k_stride + (size_t)kvh * HD);
+    const char* const v_origin = reinterpret_cast<const char*>(a.vt + (size_t)kvh * HD * a.vt_rows + vt_base_of(a.cu_rows, seq));
+    const size_t k_row_bytes = (size_t)a.k_stride * sizeof(bf16_t), v_row_bytes = (size_t)a.vt_rows * sizeof(bf16_t);
+    unsigned koff[K_EVEN ? 1 : KTASKS];
+    int kkey[K_EVEN ? 1 : KTASKS];
+#pragma unroll
+    for (int t = 0; t < (K_EVEN ? 1 : KTASKS); t++) {
+        const int i = tid + t * PTH, key = i / NCH, ch = i % NCH;
+        kkey[t] = i < PKEYS * NCH ? key : PKEYS;                    // PKEYS: no round needs it
+        koff[t] = (unsigned)(key * (int)k_row_bytes + ch * 16);
+    }
+    const int v_d = tid / VCH, v_part = tid % VCH, v_tile_key = (v_part >> 2) * BKV;     // task t: head element v_d + t * PTH / VCH
+    const unsigned voff = (unsigned)(v_d * (int)v_row_bytes + v_part * 16);
     auto fetch = [&](int kt) {
+        const int left = min(k_hi - kt, PKEYS);                     // keys of the round that some query sees
+        const char* const kb = k_origin + (size_t)kt * k_row_bytes;
+        const char* const vb = v_origin + (size_t)kt * sizeof(bf16_t);
 #pragma unroll
         for (int t = 0; t < KTASKS; t++) {
-            const int i = tid + t * PTH;
-            const int key = i / NCH, ch = i % NCH, tk = kt + key;
-            fk[t].u = make_uint4(0, 0, 0, 0);
-            if (i < PKEYS * NCH && tk < k_hi)
-                fk[t].u = *reinterpret_cast<const uint4*>(a.k + (size_t)(row0 + tk) * a.k_stride + (size_t)kvh * HD + ch * 8);
+            unsigned off;
+            if constexpr (K_EVEN) off = kkey[0] + t * (PTH / NCH) < left ? koff[0] + (unsigned)(t * (PTH / NCH)) * (unsigned)k_row_bytes : 0u;
+            else off = kkey[t] < left ? koff[t] : 0u;
+            fk[t] = *reinterpret_cast<const bf16x8*>(kb + off);
         }
 #pragma unroll
         for (int t = 0; t < VTASKS; t++) {
-            const int i = tid + t * PTH;
-            const int d = i / VCH, part = i % VCH;
-            fv[t].u = make_uint4(0, 0, 0, 0);
-            if (i < HD * VCH && kt + (part >> 2) * BKV < k_hi)       // a tile past the block's last key is never used
-                fv[t].u = *reinterpret_cast<const uint4*>(a.vt + ((size_t)kvh * HD + d) * a.vt_rows + vbase + kt + part * 8);
+            const bool need = v_d + t * (PTH / VCH) < HD && v_tile_key < left;      // a tile past the block's last key is never used
+            fv[t] = *reinterpret_cast<const bf16x8*>(vb + (need ? voff + (unsigned)(t * (PTH / VCH)) * (unsigned)v_row_bytes : 0u));
         }
     };
     auto stage = [&]() {
@@ -203,14 +222,14 @@ attn_prefill_k(PrefillArgs a) {
             const int i = tid + t * PTH;
             const int key = i / NCH;
             if (i < PKEYS * NCH)
-                *reinterpret_cast<uint4*>(Ks_all + (key / BKV) * KS_ELEMS + k_at(key % BKV, (i % NCH) * 8)) = fk[t].u;
+                *reinterpret_cast<bf16x8*>(Ks_all + (key / BKV) * KS_ELEMS + k_at(key % BKV, (i % NCH) * 8)) = fk[t];
         }
 #pragma unroll
         for (int t = 0; t < VTASKS; t++) {
             const int i = tid + t * PTH;
             const int d = i / VCH, part = i % VCH;                   // slots part*8 .. +7 of the round: tile part / 4
             if (i < HD * VCH)
-                *reinterpret_cast<uint4*>(Vt_all + (part >> 2) * VT_ELEMS + v_at(d, part & 3)) = fv[t].u;
+                *reinterpret_cast<bf16x8*>(Vt_all + (part >> 2) * VT_ELEMS + v_at(d, part & 3)) = fv[t];
         }
     };
     fetch(k_lo);
@@ -234,51 +253,52 @@ attn_prefill_k(PrefillArgs a) {
                 s[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qf[ks], s[j], 0, 0, 0);
             }
         }
-        // lane holds the scores of keys kt + j*16 + g*4 + i for its query qpos
-        // a tile every query of the wave sees whole needs no mask (wave-uniform)
+        // A lane holds the scores of keys kt + j*16 + g*4 + i for its query qpos.  From here on they are in units of
+        // log 2 (the constants carry the factor), so that every exponential is one instruction; the branches are the
+        // same for the whole wave.
+        float sc[8];
+        if (a.cap > 0.f) {                           // cap * tanh(x) = cap - 2 cap / (1 + e^(2x))
+#pragma unroll
+            for (int e = 0; e < 8; e++)
+                sc[e] = __builtin_fmaf(__builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(s[e >> 2][e & 3] * tanh_in)), -2.f * cap2, cap2);
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; e++) sc[e] = s[e >> 2][e & 3] * scale2;
+        }
+        // a tile every query of the wave sees whole needs no mask
         const bool whole = kt + BKV - 1 <= qw0 && qw0 + 15 < T && (a.window <= 0 || qw0 + 15 - kt < a.window);
-        float mx = -INFINITY;
+        if (!whole) {
+            const int first = kt + g * 4 - seen_lo;
 #pragma unroll
-        for (int j = 0; j < 2; j++)
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                float v = score_of(s[j][i], a.scale, a.cap, soc);
-                if (!whole) {
-                    const int tk = kt + j * 16 + g * 4 + i;
-                    const bool ok = tk <= qpos && tk < T && (a.window <= 0 || qpos - tk < a.window);
-                    v = ok ? v : -INFINITY;
-                }
-                s[j][i] = v;
-                mx = fmaxf(mx, v);
-            }
+            for (int e = 0; e < 8; e++)
+                sc[e] = (unsigned)(first + (e >> 2) * 16 + (e & 3)) <= seen_span ? sc[e] : -INFINITY;
+        }
+        float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
         mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
         const float m_new = fmaxf(m_i, mx);
-        float alpha = 1.f, sum = 0.f;
+        const float m_ref = m_new == -INFINITY ? 0.f : m_new;      // a query that has seen no key yet: every term is 0
+        const float alpha = m_i == m_new ? 1.f : __builtin_amdgcn_exp2f(m_i - m_ref);
+        float sum = 0.f;
         Frag pf;
-        if (m_new == -INFINITY) {
-            pf.u = make_uint4(0, 0, 0, 0);
-        } else {
-            alpha = __expf(m_i - m_new);
 #pragma unroll
-            for (int j = 0; j < 2; j++)
-#pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const float p = __expf(s[j][i] - m_new);
-                    sum += p;
-                    pf.h[j * 4 + i] = bf16_bits(p);
-                }
+        for (int e = 0; e < 8; e++) {
+            const float p = __builtin_amdgcn_exp2f(sc[e] - m_ref);
+            sum += p;
+            pf.h[e] = bf16_bits(p);
         }
         sum += __shfl_xor(sum, 16, 64);
         sum += __shfl_xor(sum, 32, 64);
         l_i = l_i * alpha + sum;
         m_i = m_new;
-        const bool rescale = __any(alpha != 1.f);              // once the running maxima settle, nothing to rescale
+        if (__any(alpha != 1.f)) {                   // once the running maxima settle, nothing to rescale
+#pragma unroll
+            for (int dt = 0; dt < HD / 16; dt++) o[dt] = o[dt] * alpha;
+        }
 #pragma unroll
         for (int dt = 0; dt < HD / 16; dt++) {
             Frag vf;
             vf.u = *reinterpret_cast<const uint4*>(Vt + v_at(dt * 16 + c, g));
-            if (rescale) o[dt] = o[dt] * alpha;
             o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf.v, o[dt], 0, 0, 0);
         }
     }
@@ -297,7 +317,7 @@ attn_prefill_k(PrefillArgs a) {
     float m = m_i;
 #pragma unroll
     for (int j = 0; j < PGROUPS - 1; j++) m = fmaxf(m, merge[(size_t)j * MERGE_GROUP + HD / 4]);
-    const float a0 = m_i == -INFINITY ? 0.f : __expf(m_i - m);
+    const float a0 = m_i == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m_i - m);
     float l = l_i * a0;
 #pragma unroll
     for (int dt = 0; dt < HD / 16; dt++) o[dt] = o[dt] * a0;
@@ -305,7 +325,7 @@ attn_prefill_k(PrefillArgs a) {
     for (int j = 0; j < PGROUPS - 1; j++) {
         const float* theirs = merge + (size_t)j * MERGE_GROUP;
         const float mj = theirs[HD / 4];
-        const float aj = mj == -INFINITY ? 0.f : __expf(mj - m);
+        const float aj = mj == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mj - m);
         l += theirs[HD / 4 + 1] * aj;
 #pragma unroll
         for (int dt = 0; dt < HD / 16; dt++) o[dt] = o[dt] + *reinterpret_cast<const f32x4*>(theirs + dt * 4) * aj;
@@ -348,6 +368,8 @@ extern "C" int tp_attn_prefill(const void* q, long q_stride, const void* k, long
                (uintptr_t)k % 16 == 0 && (uintptr_t)v % 16 == 0, "attention prefill: rows must be 16-byte aligned");
     TP_REQUIRE(n_seq <= 65535 && (long)tp_cdiv(max_count, 32) * H < (1L << 31), "attention prefill: %d heads / %d sequences exceed one launch", H, n_seq);
     TP_REQUIRE(workspace && (uintptr_t)workspace % 16 == 0, "attention prefill: needs its 16-byte aligned workspace");
+    TP_REQUIRE(k_stride < (1L << 22) && (long)HD * ((long)M + (long)BKV * n_seq + BKV) < (1L << 30),
+               "attention prefill: %d rows of stride %ld exceed the kernel's 32-bit offsets", M, k_stride);
     TP_REQUIRE(KV <= 65535, "attention prefill: %d kv heads exceed one launch", KV);
     const long vt_rows = (long)M + (long)BKV * n_seq + BKV;         // every sequence's region is padded to whole groups
     v_transpose_k<<<dim3(tp_cdiv(max_count, BKV), KV, n_seq), 256, 0, (hipStream_t)stream>>>(
