@@ -18,6 +18,12 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
 namespace {
 constexpr int BK = 64, LDS = BK;                              // LDS row stride in elements (128 bytes, unpadded)
 union Frag { uint4 u; bf16x8 v; };
+// The value as it is, in a vector register the compiler takes to be new: an address 'block-wide pointer + this' then
+// stays a scalar base with a 32-bit lane offset, instead of a 64-bit pointer per lane that is kept and moved along.
+__device__ __forceinline__ unsigned in_register(unsigned v) {
+    asm volatile("" : "+v"(v));
+    return v;
+}
 }
 
 // TM x TN: the 16 x 16 tiles of a wave; the block's 2 x 2 waves cover BM = 32 TM rows of X and BN = 32 TN rows of W
@@ -36,30 +42,49 @@ gemm_mfma_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __
     const int k_end = min(K, k_begin + k_per_split);
     if (gridDim.y > 1) Y = (float*)Y + (size_t)blockIdx.y * M * N;
 
-    // global -> register staging: TM (TN) chunks of 16 bytes per thread and operand; chunk c: row c / 8, k chunk c % 8
-    Frag ra[TM], rb[TN];
+    // global -> register staging: TM (TN) chunks of 16 bytes per thread and operand; chunk c = tid + 256 i: row c / 8,
+    // k chunk c % 8.  A whole k step of a whole tile is loaded without a branch or an address computed per lane: the
+    // lane's chunk 0 lies at one byte offset, fixed for the kernel, from base pointers that are the same for the whole
+    // block (32 rows on per chunk, 64 elements on per step: scalar work).  Tiles over the edge of Y and a last,
+    // partial step test every chunk.
+    bf16x8 ra[TM], rb[TN];
+    const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+    const bool inner = m0 + BM <= M && n0 + BN <= N;
+    const unsigned xoff = (unsigned)(tid >> 3) * (unsigned)K * 2u + (unsigned)(tid & 7) * 16u;      // the same for X and W
+    const size_t rows32 = (size_t)32 * K * 2;
+    const char* const x_origin = reinterpret_cast<const char*>(X + (size_t)m0 * K);
+    const char* const w_origin = reinterpret_cast<const char*>(W + (size_t)n0 * K);
     auto fetch = [&](int k0) {
+        if (inner && k0 + BK <= k_end) {
+            const char* const xb = x_origin + (size_t)k0 * 2, * const wb = w_origin + (size_t)k0 * 2;
+            const unsigned off = in_register(xoff);
 #pragma unroll
-        for (int i = 0; i < TM; i++) {
-            const int c = tid + i * 256, row = c >> 3, k = k0 + (c & 7) * 8, m = m0 + row;
-            ra[i].u = (m < M && k < k_end) ? *reinterpret_cast<const uint4*>(X + (size_t)m * K + k) : make_uint4(0, 0, 0, 0);
-        }
+            for (int i = 0; i < TM; i++) ra[i] = *reinterpret_cast<const bf16x8*>(xb + i * rows32 + off);
 #pragma unroll
-        for (int i = 0; i < TN; i++) {
-            const int c = tid + i * 256, row = c >> 3, k = k0 + (c & 7) * 8, n = n0 + row;
-            rb[i].u = (n < N && k < k_end) ? *reinterpret_cast<const uint4*>(W + (size_t)n * K + k) : make_uint4(0, 0, 0, 0);
+            for (int i = 0; i < TN; i++) rb[i] = *reinterpret_cast<const bf16x8*>(wb + i * rows32 + off);
+        } else {
+#pragma unroll
+            for (int i = 0; i < TM; i++) {
+                const int c = tid + i * 256, row = c >> 3, k = k0 + (c & 7) * 8, m = m0 + row;
+                ra[i] = (m < M && k < k_end) ? *reinterpret_cast<const bf16x8*>(X + (size_t)m * K + k) : zero;
+            }
+#pragma unroll
+            for (int i = 0; i < TN; i++) {
+                const int c = tid + i * 256, row = c >> 3, k = k0 + (c & 7) * 8, n = n0 + row;
+                rb[i] = (n < N && k < k_end) ? *reinterpret_cast<const bf16x8*>(W + (size_t)n * K + k) : zero;
+            }
         }
     };
     auto stage = [&]() {
 #pragma unroll
         for (int i = 0; i < TM; i++) {
             const int c = tid + i * 256, row = c >> 3, kc = ((c & 7) ^ (row & 7)) * 8;    // chunk j of a row sits at j ^ (row & 7)
-            *reinterpret_cast<uint4*>(As + row * LDS + kc) = ra[i].u;
+            *reinterpret_cast<bf16x8*>(As + row * LDS + kc) = ra[i];
         }
 #pragma unroll
         for (int i = 0; i < TN; i++) {
             const int c = tid + i * 256, row = c >> 3, kc = ((c & 7) ^ (row & 7)) * 8;
-            *reinterpret_cast<uint4*>(Bs + row * LDS + kc) = rb[i].u;
+            *reinterpret_cast<bf16x8*>(Bs + row * LDS + kc) = rb[i];
         }
     };
 
@@ -181,6 +206,7 @@ static void mfma_launch_tile(const GemmArgs& a, Tile t, void* y, int out_dtype, 
 int gemm_mfma_launch(const GemmArgs& a) {
     TP_REQUIRE(gemm_mfma_supports(a), "tiled product: needs bf16 and K a multiple of 8 (K=%d)", a.K);
     TP_REQUIRE(((uintptr_t)a.x % 16 == 0) && ((uintptr_t)a.w % 16 == 0), "tiled product: operands must be 16-byte aligned");
+    TP_REQUIRE(a.K < (1 << 22), "tiled product: K=%d exceeds the kernel's 32-bit offsets", a.K);
     TP_REQUIRE((long)tp_cdiv(a.M, 64) * tp_cdiv(a.N, 64) < (1L << 31), "tiled product: too many tiles for one launch (M=%d N=%d)", a.M, a.N);
     const Tile t = pick_tile(a);
     const int splits = gemm_mfma_splits(a);
