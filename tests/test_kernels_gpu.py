@@ -64,7 +64,8 @@ def test_add_rms_norm(ops, dt, post, nxt, m, d):
         assert got is None
 
 
-@pytest.mark.parametrize("m,n,k", [(8, 2304, 2048), (3, 600, 9216), (64, 2304, 4096), (700, 2304, 2048), (300, 520, 4104)])
+@pytest.mark.parametrize("m,n,k", [(8, 2304, 2048), (3, 600, 9216), (64, 2304, 4096), (700, 2304, 2048), (300, 520, 4104),
+                                   (2048, 2304, 4096)])
 def test_deferred_product_into_add_rms_norm(ops, m, n, k):
     """A product left in K slices and added by add_rms_norm equals the product, then the norm."""
     from trapetum_amd.kernels.ops import SplitRows
@@ -95,7 +96,7 @@ LINEAR_SHAPES = [(1, 16, 8), (3, 100, 72), (17, 331, 88), (64, 130, 2304), (5, 2
 LINEAR_SHAPES += [(65, 100, 64), (300, 257, 576), (1000, 520, 192), (513, 2304, 2048)]
 
 
-@pytest.mark.parametrize("algo", [1, 2, 3, 6])
+@pytest.mark.parametrize("algo", [1, 2, 3, 6, 7])
 @pytest.mark.parametrize("m,n,k", LINEAR_SHAPES)
 def test_linear_bf16(ops, algo, m, n, k):
     if algo == 2 and m > 64:

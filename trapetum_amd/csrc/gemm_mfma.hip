@@ -152,41 +152,60 @@ bool gemm_mfma_supports(const GemmArgs& a) {
     return a.in_dtype == TP_BF16 && a.K % 8 == 0;
 }
 
-// Tile of a product, in 16 x 16 tiles of a wave (the block is 2 x 2 waves).  Up to 64 rows: 64 x 64, the most
-// blocks per byte of W.  Else 128 x 256 (less LDS traffic per matrix instruction; two blocks fit a CU) where the grid
-// is at least four rounds of those 512 places, so that a last, partly filled round costs little; else 128 x 128
-// (three blocks a CU).  Measured on the 2B gate/up product: 930 against 790 TFLOP/s at 8192 rows, 700 against 790
-// at 2048; at 64 rows 35 us with 64 x 64 tiles against 45 us with 128 x 128.
+// Tile of a product, in 16 x 16 tiles of a wave (the block is 2 x 2 waves), and its K slices.  Up to 64 rows:
+// 64 x 64, the most blocks per byte of W.  Else 128 x 256 (less LDS traffic per matrix instruction; two blocks fit a
+// CU) where the grid is at least four rounds of those 512 places, so that a last, partly filled round costs little;
+// else 128 x 128 or 128 x 96 (three blocks a CU).  Measured on the 2B gate/up product: 930 against 790 TFLOP/s at
+// 8192 rows, 700 against 790 at 2048; at 64 rows 35 us with 64 x 64 tiles against 45 us with 128 x 128.
 struct Tile { int tm, tn; };
-static Tile pick_tile(const GemmArgs& a) {
-    if (a.algo == 6) return {4, 8};
-    if (a.M <= 64 && !(a.M > 32 && a.N >= 32768)) return {2, 2};    // the logits of 64 rows: 250 us with 128 x 128, 275 with 64 x 64
-    // up to 256 rows of a narrow product: 128 x 128 tiles would leave most CUs idle (down at 128 rows: 44 us
-    // on 72 blocks, against 15 us at 64 rows on 576 blocks of 64 x 64)
-    if (a.M <= 256 && (long)tp_cdiv(a.M, 128) * tp_cdiv(a.N, 128) < 256) return {2, 2};    // (at 512 rows 128 x 128 wins again)
-    if ((long)tp_cdiv(a.M, 128) * tp_cdiv(a.N, 256) >= 2048) return {4, 8};
-    return {4, 4};
+struct Plan { Tile tile; int splits; };
+
+// K slices of a product of few rows, which is bound by reading W and wants every CU streaming
+static int small_tile_splits(const GemmArgs& a, long blocks) {
+    if (blocks >= 512 || a.K < 512) return 1;
+    int s = (int)tp_cdiv(640, blocks);
+    if (s > a.K / 256) s = a.K / 256;
+    if (s > 16) s = 16;
+    return s < 1 ? 1 : s;
+}
+
+// A grid that does not fill the chip's 256 CUs evenly runs as long as its fullest CU: the time of (tile, slices) is
+// taken as the most blocks a CU gets x a block's k steps (a 128 x 96 block costs 0.8 of a 128 x 128 one: fewer products,
+// more LDS traffic for each), plus what writing and reading a further float32 slice of Y costs.  In units of a
+// 128 x 128 block's k step, fitted to the 2B down product at 2,048 rows (288 tiles of 128 x 128: 184 us whole, 140 us
+// in two slices, 115 us as 384 tiles of 128 x 96 in two slices, which is exactly three blocks a CU).
+static Plan mid_tile_plan(const GemmArgs& a, bool may_slice) {
+    const double step_us = 0.64, slice_us = (double)a.M * a.N * 8 / 4.0e6;
+    Plan best{{4, 4}, 1};
+    double best_cost = 1e30;
+    for (int tn = 4; tn >= 3; tn--) {
+        if (tn == 3 && a.epilogue == TP_EPI_GATED) continue;             // gate and up columns come in pairs of tiles
+        const long tiles = (long)tp_cdiv(a.M, 128) * tp_cdiv(a.N, 32 * tn);
+        for (int s = 1; s <= (may_slice ? 4 : 1); s++) {
+            if (s > 1 && a.K / s < 512) break;
+            const double k_steps = (double)tp_cdiv(tp_cdiv(a.K, s), BK);
+            const double cost = (double)tp_cdiv(tiles * s, 256) * k_steps * step_us * (tn == 3 ? 0.8 : 1.0) + (s - 1) * slice_us;
+            if (cost < best_cost * 0.97) { best_cost = cost; best = {{4, tn}, s}; }      // a tie stays with the earlier, plainer plan
+        }
+    }
+    return best;
+}
+
+static Plan plan_of(const GemmArgs& a) {
+    const bool may_slice = a.defer && a.epilogue == TP_EPI_NONE && a.algo != 6 && a.algo != 7;
+    if (a.algo == 6) return {{4, 8}, 1};
+    if (a.algo == 7) return {{4, a.epilogue == TP_EPI_GATED ? 4 : 3}, 1};
+    // the logits of 64 rows: 250 us with 128 x 128, 275 with 64 x 64; up to 256 rows of a narrow product: 128 x 128
+    // tiles would leave most CUs idle (down at 128 rows: 44 us on 72 blocks, against 15 us at 64 rows on 576 blocks
+    // of 64 x 64; at 512 rows 128 x 128 wins again)
+    if ((a.M <= 64 && !(a.M > 32 && a.N >= 32768)) || (a.M <= 256 && (long)tp_cdiv(a.M, 128) * tp_cdiv(a.N, 128) < 256))
+        return {{2, 2}, may_slice ? small_tile_splits(a, (long)tp_cdiv(a.M, 64) * tp_cdiv(a.N, 64)) : 1};
+    if ((long)tp_cdiv(a.M, 128) * tp_cdiv(a.N, 256) >= 2048) return {{4, 8}, 1};
+    return mid_tile_plan(a, may_slice);
 }
 
 // K slices for products whose tiles alone do not fill the chip and whose consumer adds the slices (defer)
-int gemm_mfma_splits(const GemmArgs& a) {
-    if (!a.defer || a.epilogue != TP_EPI_NONE || a.algo == 6) return 1;
-    const Tile t = pick_tile(a);
-    const long blocks = (long)tp_cdiv(a.M, 32 * t.tm) * tp_cdiv(a.N, 32 * t.tn);
-    int s;
-    if (t.tm == 2) {                                    // few rows: bound by reading W, wants every CU streaming
-        if (blocks >= 512 || a.K < 512) return 1;
-        s = (int)tp_cdiv(640, blocks);
-        if (s > a.K / 256) s = a.K / 256;
-        if (s > 16) s = 16;
-    } else {
-        if (blocks >= 448 || a.K < 1024) return 1;      // measured at 288 tiles: the slices win back a fifth
-        s = (int)(640 / blocks);
-        if (s > a.K / 512) s = a.K / 512;
-        if (s > 4) s = 4;
-    }
-    return s < 1 ? 1 : s;
-}
+int gemm_mfma_splits(const GemmArgs& a) { return plan_of(a).splits; }
 
 template <int EPI, int TM, int TN>
 static void mfma_launch(const GemmArgs& a, void* y, int out_dtype, int splits, int kps) {
@@ -200,7 +219,9 @@ template <int EPI>
 static void mfma_launch_tile(const GemmArgs& a, Tile t, void* y, int out_dtype, int splits, int kps) {
     if (t.tm == 2) mfma_launch<EPI, 2, 2>(a, y, out_dtype, splits, kps);
     else if (t.tn == 8) mfma_launch<EPI, 4, 8>(a, y, out_dtype, splits, kps);
-    else mfma_launch<EPI, 4, 4>(a, y, out_dtype, splits, kps);
+    else if (t.tn == 3) {
+        if constexpr (EPI != TP_EPI_GATED) mfma_launch<EPI, 4, 3>(a, y, out_dtype, splits, kps);
+    } else mfma_launch<EPI, 4, 4>(a, y, out_dtype, splits, kps);
 }
 
 int gemm_mfma_launch(const GemmArgs& a) {
@@ -208,8 +229,9 @@ int gemm_mfma_launch(const GemmArgs& a) {
     TP_REQUIRE(((uintptr_t)a.x % 16 == 0) && ((uintptr_t)a.w % 16 == 0), "tiled product: operands must be 16-byte aligned");
     TP_REQUIRE(a.K < (1 << 22), "tiled product: K=%d exceeds the kernel's 32-bit offsets", a.K);
     TP_REQUIRE((long)tp_cdiv(a.M, 64) * tp_cdiv(a.N, 64) < (1L << 31), "tiled product: too many tiles for one launch (M=%d N=%d)", a.M, a.N);
-    const Tile t = pick_tile(a);
-    const int splits = gemm_mfma_splits(a);
+    const Plan plan = plan_of(a);
+    const Tile t = plan.tile;
+    const int splits = plan.splits;
     if (splits > 1) {
         const size_t need = (size_t)splits * a.M * a.N * sizeof(float);
         TP_REQUIRE(a.workspace && a.workspace_bytes >= need, "tiled product: workspace of %zu bytes, %zu needed", a.workspace_bytes, need);
