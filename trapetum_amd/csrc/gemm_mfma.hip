@@ -1,10 +1,10 @@
 // bf16 product for many rows (prefill): LDS-tiled, on the matrix cores, fp32 accumulation.
 //
 // Block: 256 threads = 4 waves in a 2 x 2 arrangement over a 128 x 128 (or 128 x 256) tile of Y; each wave owns
-// 64 x 64 = 4 x 4 (or 4 x 8) tiles of v_mfma_f32_16x16x32_bf16.  X rows are the A operand and W rows the B operand
+// 64 x 64 = 4 x 4 (or 4 x 8) tiles of v_mfma_f32_16x16x32_bf16.  W rows are the A operand and X rows the B operand
 // (both are contiguous along k, which is what the instruction wants per lane), so a lane ends up with
-// 4 consecutive rows of one output column, and with the gate and the up column of the same unit in two
-// accumulators of the same lane (the packed gate/up matrix alternates 16 gate rows and 16 up rows).
+// 4 consecutive columns of one row of Y (one 8- or 16-byte store), and with the gate and the up column of the same
+// unit in two accumulators of the same lane (the packed gate/up matrix alternates 16 gate rows and 16 up rows).
 // K is walked in steps of 64 through one LDS buffer; the next step's global loads are issued before the
 // current step's products and written to LDS after them.  The 16-byte chunks of an LDS row are stored at
 // chunk ^ (row & 7), so that the 16 rows a fragment read touches spread over the banks (measured: bank
@@ -112,36 +112,46 @@ gemm_mfma_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __
             for (int i = 0; i < TM; i++)
 #pragma unroll
                 for (int j = 0; j < TN; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i].v, b[j].v, acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b[j].v, a[i].v, acc[i][j], 0, 0, 0);
         }
     }
 
-    // lane holds Y[m = .. + g*4 + v][n = .. + r]
+    // lane holds Y[m = .. + r][n = .. + g*4 + v], v = 0..3: four neighbours of a row go out in one store where the
+    // row length allows the alignment
+    const int width = EPI == TP_EPI_GATED ? units : N;
+    const bool wide = (width & 3) == 0;
 #pragma unroll
     for (int i = 0; i < TM; i++) {
+        const int m = m0 + wm * 16 * TM + i * 16 + r;
+        if (m >= M) continue;
 #pragma unroll
-        for (int v = 0; v < 4; v++) {
-            const int m = m0 + wm * 16 * TM + i * 16 + g * 4 + v;
-            if (m >= M) continue;
+        for (int j = 0; j < TN; j += (EPI == TP_EPI_GATED ? 2 : 1)) {
+            float o[4];
+            int col;                                            // first of the four columns of Y (units if gated)
             if (EPI == TP_EPI_GATED) {
+                col = ((n0 + wn * 16 * TN + j * 16) >> 1) + g * 4;
 #pragma unroll
-                for (int j = 0; j < TN; j += 2) {
-                    const int unit = ((n0 + wn * 16 * TN + j * 16) >> 1) + r;
-                    if (unit < units) {
-                        const float o = gelu_tanh_f(acc[i][j][v]) * acc[i][j + 1][v];
-                        if (out_dtype == TP_F32) ((float*)Y)[(size_t)m * units + unit] = o;
-                        else ((bf16_t*)Y)[(size_t)m * units + unit] = f32_to_bf16(o);
-                    }
+                for (int v = 0; v < 4; v++) o[v] = gelu_tanh_fast(acc[i][j][v]) * acc[i][j + 1 < TN ? j + 1 : j][v];
+            } else {
+                col = n0 + wn * 16 * TN + j * 16 + g * 4;
+#pragma unroll
+                for (int v = 0; v < 4; v++) o[v] = EPI == TP_EPI_SOFTCAP ? softcap_f(acc[i][j][v], cap) : acc[i][j][v];
+            }
+            if (col >= width) continue;
+            const size_t at = (size_t)m * width + col;
+            if (wide) {                                         // width % 4 == 0 and col % 4 == 0: all four are inside
+                if (out_dtype == TP_F32) *reinterpret_cast<f32x4*>((float*)Y + at) = (f32x4){o[0], o[1], o[2], o[3]};
+                else {
+                    ushort4 pk;
+                    pk.x = f32_to_bf16(o[0]); pk.y = f32_to_bf16(o[1]); pk.z = f32_to_bf16(o[2]); pk.w = f32_to_bf16(o[3]);
+                    *reinterpret_cast<ushort4*>((bf16_t*)Y + at) = pk;
                 }
             } else {
 #pragma unroll
-                for (int j = 0; j < TN; j++) {
-                    const int n = n0 + wn * 16 * TN + j * 16 + r;
-                    if (n >= N) continue;
-                    float o = acc[i][j][v];
-                    if (EPI == TP_EPI_SOFTCAP) o = softcap_f(o, cap);
-                    if (out_dtype == TP_F32) ((float*)Y)[(size_t)m * N + n] = o;
-                    else ((bf16_t*)Y)[(size_t)m * N + n] = f32_to_bf16(o);
+                for (int v = 0; v < 4; v++) {
+                    if (col + v >= width) break;
+                    if (out_dtype == TP_F32) ((float*)Y)[at + v] = o[v];
+                    else ((bf16_t*)Y)[at + v] = f32_to_bf16(o[v]);
                 }
             }
         }

@@ -148,7 +148,7 @@ gemm_skinny_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* 
 #pragma unroll
             for (int s = 0; s + 1 < NT; s += 2) {         // tiles alternate: 16 gate rows, the 16 up rows of the same units
                 const int unit = ((n0 + s * 16) >> 1) + nl;
-                if (unit < units) store_out(Y, out_dtype, (size_t)m * units + unit, gelu_tanh_f(v[t][s]) * v[t][s + 1]);
+                if (unit < units) store_out(Y, out_dtype, (size_t)m * units + unit, gelu_tanh_fast(v[t][s]) * v[t][s + 1]);
             }
         } else {
 #pragma unroll
@@ -178,7 +178,7 @@ __global__ void skinny_reduce_k(const float* __restrict__ part, void* __restrict
                 gsum += p[ng];
                 usum += p[ng + 16];
             }
-            store_out(Y, out_dtype, idx, gelu_tanh_f(gsum) * usum);
+            store_out(Y, out_dtype, idx, gelu_tanh_fast(gsum) * usum);
         } else {
             float sum = 0.f;
             for (int s = 0; s < n_splits; s++) sum += part[((size_t)s * M + m) * N + c];
