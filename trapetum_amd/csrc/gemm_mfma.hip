@@ -27,7 +27,8 @@ __device__ __forceinline__ unsigned in_register(unsigned v) {
 }
 
 // TM x TN: the 16 x 16 tiles of a wave; the block's 2 x 2 waves cover BM = 32 TM rows of X and BN = 32 TN rows of W
-template <int EPI, int TM, int TN>
+// SHORT: whole tiles load their k steps by the short path described below
+template <int EPI, int TM, int TN, bool SHORT>
 __global__ void __launch_bounds__(256, 2)
 gemm_mfma_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __restrict__ Y,
             int M, int N, int K, int m_tiles, int out_dtype, float cap, int units, int k_per_split) {
@@ -45,11 +46,13 @@ gemm_mfma_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __
     // global -> register staging: TM (TN) chunks of 16 bytes per thread and operand; chunk c = tid + 256 i: row c / 8,
     // k chunk c % 8.  A whole k step of a whole tile is loaded without a branch or an address computed per lane: the
     // lane's chunk 0 lies at one byte offset, fixed for the kernel, from base pointers that are the same for the whole
-    // block (32 rows on per chunk, 64 elements on per step: scalar work).  Tiles over the edge of Y and a last,
-    // partial step test every chunk.
+    // block (32 rows on per chunk, 64 elements on per step: scalar work).  A tile over the edge of Y computes a clamped
+    // row per chunk; only a last, partial step tests every chunk.  A launch without a whole tile (fewer rows than a tile has) and the 64 x 64 tiles,
+    // which stream W, run without the short path compiled in: its mere presence costs them a fifth (27B gate/up at 64
+    // rows in 128 x 128 tiles: 188 against 149 us), while whole large tiles gain a twentieth from it.
     bf16x8 ra[TM], rb[TN];
     const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-    const bool inner = m0 + BM <= M && n0 + BN <= N;
+    const bool inner = SHORT && m0 + BM <= M && n0 + BN <= N;
     const unsigned xoff = (unsigned)(tid >> 3) * (unsigned)K * 2u + (unsigned)(tid & 7) * 16u;      // the same for X and W
     const size_t rows32 = (size_t)32 * K * 2;
     const char* const x_origin = reinterpret_cast<const char*>(X + (size_t)m0 * K);
@@ -62,6 +65,16 @@ gemm_mfma_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __
             for (int i = 0; i < TM; i++) ra[i] = *reinterpret_cast<const bf16x8*>(xb + i * rows32 + off);
 #pragma unroll
             for (int i = 0; i < TN; i++) rb[i] = *reinterpret_cast<const bf16x8*>(wb + i * rows32 + off);
+        } else if (SHORT && k0 + BK <= k_end) {
+            // a tile over the edge of Y: a row past the edge reads the tile's last row (its products are never stored)
+            const char* const xb = x_origin + (size_t)k0 * 2, * const wb = w_origin + (size_t)k0 * 2;
+            const unsigned chunk = in_register((unsigned)(tid & 7) * 16u), row_bytes = (unsigned)K * 2u;
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+                ra[i] = *reinterpret_cast<const bf16x8*>(xb + ((unsigned)min((tid >> 3) + 32 * i, M - 1 - m0) * row_bytes + chunk));
+#pragma unroll
+            for (int i = 0; i < TN; i++)
+                rb[i] = *reinterpret_cast<const bf16x8*>(wb + ((unsigned)min((tid >> 3) + 32 * i, N - 1 - n0) * row_bytes + chunk));
         } else {
 #pragma unroll
             for (int i = 0; i < TM; i++) {
@@ -221,8 +234,12 @@ template <int EPI, int TM, int TN>
 static void mfma_launch(const GemmArgs& a, void* y, int out_dtype, int splits, int kps) {
     const int m_tiles = tp_cdiv(a.M, 32 * TM), n_tiles = tp_cdiv(a.N, 32 * TN);
     dim3 grid((unsigned)(m_tiles * n_tiles), splits);
-    gemm_mfma_k<EPI, TM, TN><<<grid, 256, 0, a.stream>>>((const bf16_t*)a.x, (const bf16_t*)a.w, y, a.M, a.N, a.K, m_tiles,
-                                                         out_dtype, a.cap, a.units, kps);
+    if (TM > 2 && a.M >= 32 * TM && a.N >= 32 * TN)
+        gemm_mfma_k<EPI, TM, TN, (TM > 2)><<<grid, 256, 0, a.stream>>>((const bf16_t*)a.x, (const bf16_t*)a.w, y, a.M, a.N, a.K, m_tiles,
+                                                                      out_dtype, a.cap, a.units, kps);
+    else
+        gemm_mfma_k<EPI, TM, TN, false><<<grid, 256, 0, a.stream>>>((const bf16_t*)a.x, (const bf16_t*)a.w, y, a.M, a.N, a.K, m_tiles,
+                                                                   out_dtype, a.cap, a.units, kps);
 }
 
 template <int EPI>
