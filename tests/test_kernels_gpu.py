@@ -149,6 +149,26 @@ def test_gated_linear(ops, algo, dt, m, inter, k):
     assert rel_l2(got, ref) < (5e-6 if dt == "f32" else 4e-3)
 
 
+@pytest.mark.parametrize("algo,m", [(2, 8), (3, 8), (3, 200)])
+def test_gated_linear_at_the_ends_of_the_activation(ops, algo, m):
+    """Gate values far out on both sides (the activation is the identity on one, zero on the other): no overflow of the
+    exponential shows in the result."""
+    k, inter = 64, 96
+    wg, wu = randn(inter, k, dtype=torch.bfloat16, seed=14), randn(inter, k, dtype=torch.bfloat16, seed=15, scale=0.2)
+    x = randn(m, k, dtype=torch.bfloat16, seed=16)
+    x[::2] *= 1.0e4
+    x[1::4] *= 1.0e15
+    ops.force_linear = algo
+    try:
+        got = ops.gated_linear(x, ops.pack_gate_up(wg, wu), inter, "gelu_tanh", torch.float32)
+    finally:
+        ops.force_linear = 0
+    g, u = x.cpu().double() @ wg.cpu().double().T, x.cpu().double() @ wu.cpu().double().T
+    ref = torch.nn.functional.gelu(g, approximate="tanh") * u
+    assert torch.isfinite(got).all()
+    assert rel_l2(got, ref) < 1e-5
+
+
 # ---- RoPE + cache write, attention over pages --------------------------------------------------------------
 def build_cache_case(dt, H, KV, hd, lens, page, rows_cap, n_pages, seed):
     """Random q/k/v rows for sequences of the given lengths, pushed through rope_kv_write of the reference."""
