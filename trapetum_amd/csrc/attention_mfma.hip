@@ -378,9 +378,15 @@ extern "C" int tp_attn_prefill(const void* q, long q_stride, const void* k, long
     PrefillArgs a{(const bf16_t*)q, q_stride, (const bf16_t*)k, k_stride, (const bf16_t*)v, v_stride, H, KV, cu_rows,
                   scale, cap, window, (bf16_t*)out, (const bf16_t*)workspace, vt_rows};
     // 64 queries a block stage each key once per 64 queries; 32 a block make twice the blocks, for grids that would
-    // leave CUs idle behind the longest tiles (measured at 2,048 tokens: 8 heads of 256 93 against 103 us with 32
-    // queries, 32 heads of 128 186 against 116 us)
-    const bool small = (long)tp_cdiv(max_count, 64) * H * n_seq <= 384;
+    // not give every CU a block of 64 (measured, 8 heads of 256: 26 against 30 us at 512 tokens, 75 against 84 at
+    // 2,048, but 151 against 121 at 3,072; 32 heads of 128 at 2,048 tokens: 145 against 89 us)
+    static int cus = 0;
+    if (!cus) {
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+            cus = 256;
+    }
+    const bool small = (long)tp_cdiv(max_count, 64) * H * n_seq <= cus;
     if (int rc = small ? prefill_launch<32>(a, max_count, H, n_seq, (hipStream_t)stream)
                        : prefill_launch<64>(a, max_count, H, n_seq, (hipStream_t)stream)) return rc;
     return tp_check_launch("attention prefill");
