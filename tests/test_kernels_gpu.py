@@ -194,15 +194,18 @@ def build_cache_case(dt, H, KV, hd, lens, page, rows_cap, n_pages, seed):
 @pytest.mark.parametrize("dt", ["f32", "bf16"])
 @pytest.mark.parametrize("H,KV,hd,lens,page,rows_cap", [
     (4, 2, 16, (5, 11, 17), 16, 0), (6, 1, 32, (1, 9, 23, 40), 16, 16), (3, 3, 48, (70, 3), 64, 64),
-    (8, 4, 256, (130,), 64, 0), (2, 2, 80, (33, 50), 16, 32), (4, 2, 64, (200, 90), 16, 0), (5, 1, 32, (300,), 16, 64)])
+    (8, 4, 256, (130,), 64, 0), (2, 2, 80, (33, 50), 16, 32), (4, 2, 64, (200, 90), 16, 0), (5, 1, 32, (300,), 16, 64),
+    (2, 2, 80, (150, 140), 16, 0), (8, 4, 256, (300, 77), 64, 128)])
 def test_rope_kv_write(ops, dt, H, KV, hd, lens, page, rows_cap):
     c = build_cache_case(DT[dt], H, KV, hd, lens, page, rows_cap, 24, 20)
+    rot = hd if hd != 80 else 48                            # one head size with a rotation over part of the head
+    c["inv_freq"] = c["inv_freq"][:rot // 2].contiguous()
     pools_ref = [torch.zeros(24, KV, page, hd, dtype=DT[dt]) for _ in range(2)]
     pools = [p.to(DEV) for p in pools_ref]
     q_ref, k_ref = c["q"].cpu().clone(), c["k"].cpu().clone()
-    ref_ops.rope_kv_write(q_ref, k_ref, c["v"].cpu(), H, KV, hd, c["inv_freq"], hd, c["row_seq"], c["row_pos"],
+    ref_ops.rope_kv_write(q_ref, k_ref, c["v"].cpu(), H, KV, hd, c["inv_freq"], rot, c["row_seq"], c["row_pos"],
                           c["new_len"], c["table"], pools_ref[0], pools_ref[1], rows_cap)
-    ops.rope_kv_write(c["q"], c["k"], c["v"], H, KV, hd, c["inv_freq"].to(DEV), hd, c["row_seq"].to(DEV),
+    ops.rope_kv_write(c["q"], c["k"], c["v"], H, KV, hd, c["inv_freq"].to(DEV), rot, c["row_seq"].to(DEV),
                       c["row_pos"].to(DEV), c["new_len"].to(DEV), c["table"].to(DEV), pools[0], pools[1], rows_cap)
     t = 3e-6 if dt == "f32" else 6e-3
     assert rel_l2(c["q"], q_ref) < t and rel_l2(c["k"], k_ref) < t
