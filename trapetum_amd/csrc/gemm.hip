@@ -109,16 +109,18 @@ static int pick(const GemmArgs& a, int algo) {
     if (algo == 2) return gemm_skinny_supports(a) ? 2 : -2;
     if (algo == 3 || algo == 6 || algo == 7) return gemm_mfma_supports(a) ? 3 : -3;
     // Up to 64 rows both matrix-core kernels stream W once; which is faster was measured on MI355X at the 2B shapes
-    // (cold weights, microseconds, skinny / tiled with 64 x 64 tiles):
+    // (cold weights, microseconds, skinny / tiled with 64 x 64 tiles and k steps of 128):
     //   logits  N 256000            8 rows 277 / 222
-    //   down    N 2304  K 9216      1 row 13.1 / 12.7    8 rows 15.4 / 13.1    64 rows 25.9 / 15.4   (K slices left to the consumer)
-    //   qkv     N 4096  K 2304      1 row  6.9 /  6.5    8 rows  7.5 /  6.9    64 rows 13.2 /  8.7   (K slices)
-    //   o       N 2304  K 2048      8 rows  5.2 /  6.0   16 rows  5.8 /  6.1   24 rows  7.0 /  6.6   (K slices)
-    //   gate/up N 18432 K 2304      8 rows 26.6 / 33.5   16 rows 30.6 / 33.5   24 rows 40.8 / 34.6   (no slices: gated)
+    //   down    N 2304  K 9216      8 rows 15.8 / 11.3   32 rows 20.1 / 12.0   64 rows 26.3 / 13.5   (K slices left to the consumer)
+    //   qkv     N 4096  K 2304      8 rows  8.0 /  7.1   32 rows 11.7 /  7.5   64 rows 13.5 /  8.5   (K slices)
+    //   o       N 2304  K 2048      8 rows  5.2 /  5.5   32 rows  7.7 /  6.0   64 rows 13.3 /  6.7   (K slices)
+    //   gate/up N 18432 K 2304      8 rows 26.9 / 24.2   32 rows 40.7 / 24.7   64 rows 48.5 / 26.5   (no slices: gated)
     if (gemm_mfma_supports(a)) {
         const bool sliced = a.defer && a.epilogue == TP_EPI_NONE;
         // (up to 16 rows the tiled kernel's lead on qkv and down is lost again in their consumers, which then add
-        // 9 and 16 slices instead of 2 and 4: a decode step of 8 sequences took 2.44 ms instead of 2.36)
+        // 9 and 16 slices instead of 2 and 4: a decode step of 8 sequences took 2.40 ms instead of 2.26; a single
+        // sequence is faster on the skinny kernel throughout)
+        if (a.M >= 8 && a.epilogue == TP_EPI_GATED) return 3;
         if (a.M >= 8 && a.N >= 32768) return 3;
         if (a.M > 16 && (sliced || a.N >= 8192)) return 3;
     }

@@ -16,7 +16,11 @@ typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
 
 namespace {
-constexpr int BK = 64, LDS = BK;                              // LDS row stride in elements (128 bytes, unpadded)
+constexpr int BK = 64;                                        // k step of the large tiles; LDS rows are one step long, unpadded
+// k step of the 64 x 64 tiles.  They stream W, and what a block has in flight is one step of its tile: with steps of
+// 64 the 288 blocks of the 2B gate/up product hold 2.4 MB between them, too little to keep HBM busy (cold weights,
+// 64 rows: 34.6 us; steps of 128: 26.4 us; steps of 256: 26.3 us, and the smaller products lose).
+constexpr int SMALL_KS = 128;
 union Frag { uint4 u; bf16x8 v; };
 // The value as it is, in a vector register the compiler takes to be new: an address 'block-wide pointer + this' then
 // stays a scalar base with a 32-bit lane offset, instead of a 64-bit pointer per lane that is kept and moved along.
@@ -28,11 +32,14 @@ __device__ __forceinline__ unsigned in_register(unsigned v) {
 
 // TM x TN: the 16 x 16 tiles of a wave; the block's 2 x 2 waves cover BM = 32 TM rows of X and BN = 32 TN rows of W
 // SHORT: whole tiles load their k steps by the short path described below
-template <int EPI, int TM, int TN, bool SHORT>
+// KS: elements of a k step (64, or 128 for the 64 x 64 tiles, which stream W and are bound by the bytes a block has
+// in flight: one step ahead is all a block asks for)
+template <int EPI, int TM, int TN, bool SHORT, int KS = BK>
 __global__ void __launch_bounds__(256, 2)
 gemm_mfma_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __restrict__ Y,
             int M, int N, int K, int m_tiles, int out_dtype, float cap, int units, int k_per_split) {
-    constexpr int BM = 32 * TM, BN = 32 * TN;
+    constexpr int BM = 32 * TM, BN = 32 * TN, BK = KS, LDS = KS, CPR = KS / 8, LA = TM * KS / 64, LB = TN * KS / 64;
+    static_assert(!SHORT || KS == 64, "the short load path is written for steps of 64");
     __shared__ __attribute__((aligned(16))) bf16_t As[BM * LDS];
     __shared__ __attribute__((aligned(16))) bf16_t Bs[BN * LDS];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 15, g = lane >> 4;
@@ -50,7 +57,7 @@ gemm_mfma_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __
     // row per chunk; only a last, partial step tests every chunk.  A launch without a whole tile (fewer rows than a tile has) and the 64 x 64 tiles,
     // which stream W, run without the short path compiled in: its mere presence costs them a fifth (27B gate/up at 64
     // rows in 128 x 128 tiles: 188 against 149 us), while whole large tiles gain a twentieth from it.
-    bf16x8 ra[TM], rb[TN];
+    bf16x8 ra[LA], rb[LB];
     const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
     const bool inner = SHORT && m0 + BM <= M && n0 + BN <= N;
     const unsigned xoff = (unsigned)(tid >> 3) * (unsigned)K * 2u + (unsigned)(tid & 7) * 16u;      // the same for X and W
@@ -77,26 +84,26 @@ gemm_mfma_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __
                 rb[i] = *reinterpret_cast<const bf16x8*>(wb + ((unsigned)min((tid >> 3) + 32 * i, N - 1 - n0) * row_bytes + chunk));
         } else {
 #pragma unroll
-            for (int i = 0; i < TM; i++) {
-                const int c = tid + i * 256, row = c >> 3, k = k0 + (c & 7) * 8, m = m0 + row;
+            for (int i = 0; i < LA; i++) {
+                const int c = tid + i * 256, row = c / CPR, k = k0 + (c % CPR) * 8, m = m0 + row;
                 ra[i] = (m < M && k < k_end) ? *reinterpret_cast<const bf16x8*>(X + (size_t)m * K + k) : zero;
             }
 #pragma unroll
-            for (int i = 0; i < TN; i++) {
-                const int c = tid + i * 256, row = c >> 3, k = k0 + (c & 7) * 8, n = n0 + row;
+            for (int i = 0; i < LB; i++) {
+                const int c = tid + i * 256, row = c / CPR, k = k0 + (c % CPR) * 8, n = n0 + row;
                 rb[i] = (n < N && k < k_end) ? *reinterpret_cast<const bf16x8*>(W + (size_t)n * K + k) : zero;
             }
         }
     };
     auto stage = [&]() {
 #pragma unroll
-        for (int i = 0; i < TM; i++) {
-            const int c = tid + i * 256, row = c >> 3, kc = ((c & 7) ^ (row & 7)) * 8;    // chunk j of a row sits at j ^ (row & 7)
+        for (int i = 0; i < LA; i++) {
+            const int c = tid + i * 256, row = c / CPR, kc = ((c % CPR) ^ (row & 7)) * 8;  // chunk j of a row sits at j ^ (row & 7)
             *reinterpret_cast<bf16x8*>(As + row * LDS + kc) = ra[i];
         }
 #pragma unroll
-        for (int i = 0; i < TN; i++) {
-            const int c = tid + i * 256, row = c >> 3, kc = ((c & 7) ^ (row & 7)) * 8;
+        for (int i = 0; i < LB; i++) {
+            const int c = tid + i * 256, row = c / CPR, kc = ((c % CPR) ^ (row & 7)) * 8;
             *reinterpret_cast<bf16x8*>(Bs + row * LDS + kc) = rb[i];
         }
     };
@@ -230,21 +237,21 @@ static Plan plan_of(const GemmArgs& a) {
 // K slices for products whose tiles alone do not fill the chip and whose consumer adds the slices (defer)
 int gemm_mfma_splits(const GemmArgs& a) { return plan_of(a).splits; }
 
-template <int EPI, int TM, int TN>
+template <int EPI, int TM, int TN, int KS = BK>
 static void mfma_launch(const GemmArgs& a, void* y, int out_dtype, int splits, int kps) {
     const int m_tiles = tp_cdiv(a.M, 32 * TM), n_tiles = tp_cdiv(a.N, 32 * TN);
     dim3 grid((unsigned)(m_tiles * n_tiles), splits);
     if (TM > 2 && a.M >= 32 * TM && a.N >= 32 * TN)
-        gemm_mfma_k<EPI, TM, TN, (TM > 2)><<<grid, 256, 0, a.stream>>>((const bf16_t*)a.x, (const bf16_t*)a.w, y, a.M, a.N, a.K, m_tiles,
+        gemm_mfma_k<EPI, TM, TN, (TM > 2), KS><<<grid, 256, 0, a.stream>>>((const bf16_t*)a.x, (const bf16_t*)a.w, y, a.M, a.N, a.K, m_tiles,
                                                                       out_dtype, a.cap, a.units, kps);
     else
-        gemm_mfma_k<EPI, TM, TN, false><<<grid, 256, 0, a.stream>>>((const bf16_t*)a.x, (const bf16_t*)a.w, y, a.M, a.N, a.K, m_tiles,
+        gemm_mfma_k<EPI, TM, TN, false, KS><<<grid, 256, 0, a.stream>>>((const bf16_t*)a.x, (const bf16_t*)a.w, y, a.M, a.N, a.K, m_tiles,
                                                                    out_dtype, a.cap, a.units, kps);
 }
 
 template <int EPI>
 static void mfma_launch_tile(const GemmArgs& a, Tile t, void* y, int out_dtype, int splits, int kps) {
-    if (t.tm == 2) mfma_launch<EPI, 2, 2>(a, y, out_dtype, splits, kps);
+    if (t.tm == 2) mfma_launch<EPI, 2, 2, SMALL_KS>(a, y, out_dtype, splits, kps);
     else if (t.tn == 8) mfma_launch<EPI, 4, 8>(a, y, out_dtype, splits, kps);
     else if (t.tn == 3) {
         if constexpr (EPI != TP_EPI_GATED) mfma_launch<EPI, 4, 3>(a, y, out_dtype, splits, kps);
@@ -262,7 +269,8 @@ int gemm_mfma_launch(const GemmArgs& a) {
     if (splits > 1) {
         const size_t need = (size_t)splits * a.M * a.N * sizeof(float);
         TP_REQUIRE(a.workspace && a.workspace_bytes >= need, "tiled product: workspace of %zu bytes, %zu needed", a.workspace_bytes, need);
-        const int kps = tp_cdiv(tp_cdiv(a.K, splits), BK) * BK;
+        const int kstep = t.tm == 2 ? SMALL_KS : BK;
+        const int kps = tp_cdiv(tp_cdiv(a.K, splits), kstep) * kstep;
         mfma_launch_tile<TP_EPI_NONE>(a, t, a.workspace, TP_F32, tp_cdiv(a.K, kps), kps);
         return tp_check_launch("linear (tiled kernel, K slices)");
     }
