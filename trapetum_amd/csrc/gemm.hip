@@ -120,7 +120,9 @@ static int pick(const GemmArgs& a, int algo) {
         // (up to 16 rows the tiled kernel's lead on qkv and down is lost again in their consumers, which then add
         // 9 and 16 slices instead of 2 and 4: a decode step of 8 sequences took 2.40 ms instead of 2.26; a single
         // sequence is faster on the skinny kernel throughout)
-        if (a.M >= 8 && a.epilogue == TP_EPI_GATED) return 3;
+        // (from 8 rows on the large matrices gain more than that: 27B down, 340 MB, 93 -> 74 us; a 27B step of 8
+        // sequences 14.2 -> 13.65 ms)
+        if (a.M >= 8 && (a.epilogue == TP_EPI_GATED || (long)a.N * a.K >= 24000000)) return 3;
         if (a.M >= 8 && a.N >= 32768) return 3;
         if (a.M > 16 && (sliced || a.N >= 8192)) return 3;
     }
