@@ -94,6 +94,9 @@ LINEAR_SHAPES = [(1, 16, 8), (3, 100, 72), (17, 331, 88), (64, 130, 2304), (5, 2
 
 
 LINEAR_SHAPES += [(65, 100, 64), (300, 257, 576), (1000, 520, 192), (513, 2304, 2048)]
+# grids of more than a thousand tiles, which the tiled kernel walks in another order (per XCD, in panels): tile counts
+# that are no multiple of 8 and a last panel that is not whole
+LINEAR_SHAPES += [(300, 44177, 64), (40, 70001, 72)]
 
 
 @pytest.mark.parametrize("algo", [1, 2, 3, 6, 7])
@@ -129,7 +132,7 @@ def test_linear_f32(ops, m, n, k):
 @pytest.mark.parametrize("algo", [1, 2, 3, 6])
 @pytest.mark.parametrize("dt", ["bf16", "f32"])
 @pytest.mark.parametrize("m,inter,k", [(1, 16, 16), (4, 200, 88), (40, 320, 96), (9, 1000, 2304), (150, 72, 136),
-                                       (150, 72, 128), (700, 1000, 320)])
+                                       (150, 72, 128), (700, 1000, 320), (130, 36010, 64)])
 def test_gated_linear(ops, algo, dt, m, inter, k):
     if dt == "f32" and algo != 1:
         pytest.skip("float32 runs on the plain kernel only")

@@ -9,7 +9,8 @@
 // current step's products and written to LDS after them.  The 16-byte chunks of an LDS row are stored at
 // chunk ^ (row & 7), so that the 16 rows a fragment read touches spread over the banks (measured: bank
 // conflicts fall from a third of the LDS cycles with padded rows to a few per cent).
-// Consecutive block ids walk the M tiles of one N tile, so blocks in flight together share W tiles.
+// Consecutive block ids walk the M tiles of one N tile, so blocks in flight together share W tiles (large grids:
+// per XCD, see the kernel).
 #include "gemm.h"
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
@@ -37,14 +38,30 @@ __device__ __forceinline__ unsigned in_register(unsigned v) {
 template <int EPI, int TM, int TN, bool SHORT, int KS = BK>
 __global__ void __launch_bounds__(256, 2)
 gemm_mfma_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __restrict__ Y,
-            int M, int N, int K, int m_tiles, int out_dtype, float cap, int units, int k_per_split) {
+            int M, int N, int K, int m_tiles, int out_dtype, float cap, int units, int k_per_split, int xcd_panels) {
     constexpr int BM = 32 * TM, BN = 32 * TN, BK = KS, LDS = KS, CPR = KS / 8, LA = TM * KS / 64, LB = TN * KS / 64;
     static_assert(!SHORT || KS == 64, "the short load path is written for steps of 64");
     __shared__ __attribute__((aligned(16))) bf16_t As[BM * LDS];
     __shared__ __attribute__((aligned(16))) bf16_t Bs[BN * LDS];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 15, g = lane >> 4;
     const int wm = wave >> 1, wn = wave & 1;
-    const int m0 = (blockIdx.x % m_tiles) * BM, n0 = (blockIdx.x / m_tiles) * BN;
+    // Block ids go to the chip's 8 XCDs in turn, and each XCD has an L2 of its own.  On a large grid an XCD therefore
+    // takes a contiguous range of the tiles, walked in panels of four N tiles (M tiles of a panel one after another, its
+    // N tiles fastest), so that the blocks an XCD runs together share their W and X tiles in its L2: measured on the
+    // 2B gate/up product at 2,048 rows, 2,304 tiles: 210 -> 185 us.  (Up to some hundred tiles nothing is gained.)
+    int vb = blockIdx.x, mt, nt;
+    if (xcd_panels) {
+        const int total = gridDim.x, base = total >> 3, rem = total & 7, xcd = vb & 7;
+        vb = xcd * base + min(xcd, rem) + (vb >> 3);
+        const int n_tiles = total / m_tiles, per_panel = 4 * m_tiles, p = vb / per_panel, q = vb - p * per_panel;
+        const int width = min(4, n_tiles - p * 4);
+        nt = p * 4 + q % width;
+        mt = q / width;
+    } else {
+        mt = vb % m_tiles;
+        nt = vb / m_tiles;
+    }
+    const int m0 = mt * BM, n0 = nt * BN;
     // a K slice per blockIdx.y: slices go to Y as float32 [slices, M, N] for the consumer to add in slice order
     const int k_begin = blockIdx.y * k_per_split;
     const int k_end = min(K, k_begin + k_per_split);
@@ -241,12 +258,13 @@ template <int EPI, int TM, int TN, int KS = BK>
 static void mfma_launch(const GemmArgs& a, void* y, int out_dtype, int splits, int kps) {
     const int m_tiles = tp_cdiv(a.M, 32 * TM), n_tiles = tp_cdiv(a.N, 32 * TN);
     dim3 grid((unsigned)(m_tiles * n_tiles), splits);
+    const int xcd_panels = (long)m_tiles * n_tiles >= 1024 ? 1 : 0;
     if (TM > 2 && a.M >= 32 * TM && a.N >= 32 * TN)
         gemm_mfma_k<EPI, TM, TN, (TM > 2), KS><<<grid, 256, 0, a.stream>>>((const bf16_t*)a.x, (const bf16_t*)a.w, y, a.M, a.N, a.K, m_tiles,
-                                                                      out_dtype, a.cap, a.units, kps);
+                                                                      out_dtype, a.cap, a.units, kps, xcd_panels);
     else
         gemm_mfma_k<EPI, TM, TN, false, KS><<<grid, 256, 0, a.stream>>>((const bf16_t*)a.x, (const bf16_t*)a.w, y, a.M, a.N, a.K, m_tiles,
-                                                                   out_dtype, a.cap, a.units, kps);
+                                                                   out_dtype, a.cap, a.units, kps, xcd_panels);
 }
 
 template <int EPI>
