@@ -48,7 +48,9 @@ def test_rms_norm(ops, din, dout, m, d):
 
 @pytest.mark.parametrize("dt", ["f32", "bf16"])
 @pytest.mark.parametrize("post,nxt", [(True, True), (True, False), (False, True), (False, False)])
-@pytest.mark.parametrize("m,d", [(1, 64), (5, 88), (4, 3584)])
+@pytest.mark.parametrize("m,d", [(1, 64), (5, 88), (4, 3584),
+                                 # many rows: four elements per lane, one width for each of its forms and their edges
+                                 (130, 88), (200, 1000), (150, 2304), (140, 3072), (129, 4608), (130, 8192), (131, 8200), (130, 90)])
 def test_add_rms_norm(ops, dt, post, nxt, m, d):
     stream = randn(m, d, seed=3, scale=2.0)
     rows = randn(m, d, dtype=DT[dt], seed=4, scale=5.0)

@@ -184,11 +184,104 @@ add_rms_norm_reg_k(float* __restrict__ stream, const TR* __restrict__ rows, int 
     }
 }
 
+// The same for many rows, where the kernel is bound by the volume of its loads: a lane takes four neighbouring
+// elements per load (16 bytes of float32, 8 of bf16), CPT such chunks NTH lanes apart.  Needs D % 4 == 0.
+__device__ __forceinline__ void ld4(const float* p, float (&o)[4]) {
+    const float4 t = *reinterpret_cast<const float4*>(p);
+    o[0] = t.x; o[1] = t.y; o[2] = t.z; o[3] = t.w;
+}
+__device__ __forceinline__ void ld4(const bf16_t* p, float (&o)[4]) {
+    const uint2 t = *reinterpret_cast<const uint2*>(p);
+    o[0] = __uint_as_float(t.x << 16); o[1] = __uint_as_float(t.x & 0xffff0000u);
+    o[2] = __uint_as_float(t.y << 16); o[3] = __uint_as_float(t.y & 0xffff0000u);
+}
+__device__ __forceinline__ void st4(float* p, const float (&v)[4]) {
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+}
+__device__ __forceinline__ void st4(bf16_t* p, const float (&v)[4]) {
+    uint2 t;
+    t.x = (uint32_t)f32_to_bf16(v[0]) | ((uint32_t)f32_to_bf16(v[1]) << 16);
+    t.y = (uint32_t)f32_to_bf16(v[2]) | ((uint32_t)f32_to_bf16(v[3]) << 16);
+    *reinterpret_cast<uint2*>(p) = t;
+}
+
+template <typename TR, typename T, int CPT, int NTH>
+__global__ void __launch_bounds__(NTH)
+add_rms_norm_vec_k(float* __restrict__ stream, const TR* __restrict__ rows, int n_slices, long slice_stride,
+                   const float* __restrict__ gain_post, float eps_post,
+                   const float* __restrict__ gain_next, float eps_next, T* __restrict__ out, int D) {
+    __shared__ float red[16];
+    float* sr = stream + (size_t)blockIdx.x * D;
+    const TR* ar = rows + (size_t)blockIdx.x * D;
+    float a[CPT][4], v[CPT][4], gp[CPT][4], gn[CPT][4];
+#pragma unroll
+    for (int j = 0; j < CPT; j++) {
+        const int i = (threadIdx.x + j * NTH) * 4;
+        const bool ok = i < D;
+        const int ic = ok ? i : 0;                       // a chunk past the row reads the row's first and counts as zero
+        ld4(ar + ic, a[j]);
+        for (int sl = 1; sl < n_slices; sl++) {          // slices in slice order
+            float t[4];
+            ld4(ar + (size_t)sl * slice_stride + ic, t);
+#pragma unroll
+            for (int e = 0; e < 4; e++) a[j][e] += t[e];
+        }
+        ld4(sr + ic, v[j]);
+        if (gain_post) ld4(gain_post + ic, gp[j]);
+        if (gain_next) ld4(gain_next + ic, gn[j]);
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            if (!ok) { a[j][e] = 0.f; v[j][e] = 0.f; }
+            if (!gain_post) gp[j][e] = 1.f;
+        }
+    }
+    float scale_a = 1.f;
+    if (gain_post) {
+        float ss = 0.f;
+#pragma unroll
+        for (int j = 0; j < CPT; j++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) ss += a[j][e] * a[j][e];
+        ss = block_sum(ss, red);
+        scale_a = rsqrtf(ss / (float)D + eps_post);
+    }
+    float ss2 = 0.f;
+#pragma unroll
+    for (int j = 0; j < CPT; j++) {
+        const int i = (threadIdx.x + j * NTH) * 4;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            float t = a[j][e];
+            if (gain_post) t = (t * scale_a) * gp[j][e];
+            v[j][e] += t;
+            ss2 += v[j][e] * v[j][e];                    // chunks past the row hold zeros
+        }
+        if (i < D) st4(sr + i, v[j]);
+    }
+    if (!gain_next) return;
+    ss2 = block_sum(ss2, red);
+    const float scale_s = rsqrtf(ss2 / (float)D + eps_next);
+    T* orow = out + (size_t)blockIdx.x * D;
+#pragma unroll
+    for (int j = 0; j < CPT; j++) {
+        const int i = (threadIdx.x + j * NTH) * 4;
+        float o[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) o[e] = (v[j][e] * scale_s) * gn[j][e];
+        if (i < D) st4(orow + i, o);
+    }
+}
+
 template <typename TR, typename T>
 static int add_rms_norm_launch(float* stream, const void* rows, int n_slices, long slice_stride, const float* gp, float ep,
                                const float* gn, float en, void* out, int M, int D, hipStream_t s) {
     // few rows: many threads per row (the kernel is bound by the latency of its loads, not by their volume)
-    if (D <= 256 * 2) add_rms_norm_reg_k<TR, T, 2, 256><<<M, 256, 0, s>>>(stream, (const TR*)rows, n_slices, slice_stride, gp, ep, gn, en, (T*)out, D);
+    const bool vec = M > 128 && D % 4 == 0 && (uintptr_t)rows % 16 == 0 && (uintptr_t)stream % 16 == 0 && slice_stride % 4 == 0 &&
+                     (!gp || (uintptr_t)gp % 16 == 0) && (!gn || (uintptr_t)gn % 16 == 0) && (!out || (uintptr_t)out % 16 == 0);
+    if (vec && D <= 256 * 4) add_rms_norm_vec_k<TR, T, 1, 256><<<M, 256, 0, s>>>(stream, (const TR*)rows, n_slices, slice_stride, gp, ep, gn, en, (T*)out, D);
+    else if (vec && D <= 256 * 12) add_rms_norm_vec_k<TR, T, 3, 256><<<M, 256, 0, s>>>(stream, (const TR*)rows, n_slices, slice_stride, gp, ep, gn, en, (T*)out, D);
+    else if (vec && D <= 512 * 16) add_rms_norm_vec_k<TR, T, 4, 512><<<M, 512, 0, s>>>(stream, (const TR*)rows, n_slices, slice_stride, gp, ep, gn, en, (T*)out, D);
+    else if (D <= 256 * 2) add_rms_norm_reg_k<TR, T, 2, 256><<<M, 256, 0, s>>>(stream, (const TR*)rows, n_slices, slice_stride, gp, ep, gn, en, (T*)out, D);
     else if (M <= 128 && D <= 1024 * 4) add_rms_norm_reg_k<TR, T, 4, 1024><<<M, 1024, 0, s>>>(stream, (const TR*)rows, n_slices, slice_stride, gp, ep, gn, en, (T*)out, D);
     else if (D <= 256 * 4) add_rms_norm_reg_k<TR, T, 4, 256><<<M, 256, 0, s>>>(stream, (const TR*)rows, n_slices, slice_stride, gp, ep, gn, en, (T*)out, D);
     else if (D <= 256 * 12) add_rms_norm_reg_k<TR, T, 12, 256><<<M, 256, 0, s>>>(stream, (const TR*)rows, n_slices, slice_stride, gp, ep, gn, en, (T*)out, D);
