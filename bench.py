@@ -1,7 +1,7 @@
 """Benchmark: decode tokens per second of Gemma-2 at 2B layer sizes with random weights on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--dtype bfloat16|float32]
-                    [--sizes 2b|9b|27b] [--prompt T]
+                    [--sizes 2b|9b|27b] [--prompt T] [--batch B]
 
 A step is one decode step of a batch of 8 sequences (a token each, chosen greedily on the device and fed to
 the next step).  One JSON line is printed: decode tokens per second as `value`, the prefill of 2,048 tokens,
@@ -65,6 +65,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--sizes", default="2b", choices=sorted(OTHER_SIZES), help="layer sizes of which Gemma-2 (the metric is 2b)")
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the configuration's, if memory or time needs it")
+    ap.add_argument("--batch", type=int, default=BATCH, help="sequences of the timed decode steps (the metric: 8)")
     ap.add_argument("--prompt", type=int, default=PROMPT, help="tokens of each prompt before decoding (the metric: 512)")
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip decode at batch 1 and 64")
@@ -85,9 +86,9 @@ def main():
     cfg = Gemma2Config.from_kwargs(**dict(sizes, num_hidden_layers=args.layers or full_layers))
     itemsize = 2 if args.dtype == "bfloat16" else 4
     t0 = time.time()
-    most = max(PREFILL_TOKENS, (BATCH if args.no_points else 64) * (args.prompt + args.steps + args.warmup + 128))
+    most = max(PREFILL_TOKENS, (args.batch if args.no_points else max(64, args.batch)) * (args.prompt + args.steps + args.warmup + 128))
     engine = Engine.from_config(cfg, seed=2, sigma=0.02, dtype=args.dtype, draw_on_device=True,
-                                max_tokens_in_cache=max(64 * 1024, most), max_context=CONTEXT, max_batch=64)
+                                max_tokens_in_cache=max(64 * 1024, most), max_context=CONTEXT, max_batch=max(64, args.batch))
     model, cache = engine.model, engine.cache
     torch.cuda.synchronize()
     print(f"[bench] model ready in {time.time() - t0:.1f}s", file=sys.stderr, flush=True)
@@ -130,10 +131,10 @@ def main():
         loop.finish()
         return dt, ctx0 + steps / 2.0
 
-    dt, mean_ctx = decode(BATCH, args.steps, args.warmup)
+    dt, mean_ctx = decode(args.batch, args.steps, args.warmup)
     ms_step = dt / args.steps * 1e3
-    value = BATCH * args.steps / dt
-    step_bytes = weight_bytes(cfg, itemsize) + BATCH * kv_bytes(cfg, int(mean_ctx), itemsize)
+    value = args.batch * args.steps / dt
+    step_bytes = weight_bytes(cfg, itemsize) + args.batch * kv_bytes(cfg, int(mean_ctx), itemsize)
     achieved = step_bytes / (dt / args.steps) / 1e9
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                 "frac": round(achieved / PEAK_HBM_GBS, 4)}
@@ -145,14 +146,14 @@ def main():
             print(f"[bench] decode batch {b}: {points[f'decode_b{b}']} tok/s", file=sys.stderr, flush=True)
 
     line = {
-        "metric": f"decode tok/s @ batch 8, Gemma-2-{args.sizes.upper()} layer sizes", "value": round(value, 1), "unit": "tok/s",
+        "metric": f"decode tok/s @ batch {args.batch}, Gemma-2-{args.sizes.upper()} layer sizes", "value": round(value, 1), "unit": "tok/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
         "data": "synthetic: seeded random weights N(0, 0.02) and uniform-random token ids",
         "config": {"model": f"gemma-2-{args.sizes} sizes", "layers": cfg.num_hidden_layers, "layers_full": full_layers,
                    "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
                    "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
-                   "window": cfg.sliding_window, "global_batch": BATCH, "seq_len": CONTEXT, "prompt_len": args.prompt,
+                   "window": cfg.sliding_window, "global_batch": args.batch, "seq_len": CONTEXT, "prompt_len": args.prompt,
                    "decode_context": round(mean_ctx, 1), "hip_graph": not args.no_graph, "parallelism": "single GPU"},
         "prefill": prefill, "roofline": roofline, "points": points,
     }

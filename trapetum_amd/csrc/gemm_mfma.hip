@@ -7,7 +7,7 @@
 // unit in two accumulators of the same lane (the packed gate/up matrix alternates 16 gate rows and 16 up rows).
 // K is walked in steps of 64 through one LDS buffer; the next step's global loads are issued before the
 // current step's products and written to LDS after them.  The 16-byte chunks of an LDS row are stored at
-// chunk ^ (row & 7), so that the 16 rows a fragment read touches spread over the banks (measured: bank
+// chunk ^ (row & 7) (rows of 128 bytes; ^ (row & 15) in rows of 256), so that the 16 rows a fragment read touches spread over the banks (measured: bank
 // conflicts fall from a third of the LDS cycles with padded rows to a few per cent).
 // Consecutive block ids walk the M tiles of one N tile, so blocks in flight together share W tiles (large grids:
 // per XCD, see the kernel).
@@ -40,6 +40,7 @@ __global__ void __launch_bounds__(256, 2)
 gemm_mfma_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __restrict__ Y,
             int M, int N, int K, int m_tiles, int out_dtype, float cap, int units, int k_per_split, int xcd_panels) {
     constexpr int BM = 32 * TM, BN = 32 * TN, BK = KS, LDS = KS, CPR = KS / 8, LA = TM * KS / 64, LB = TN * KS / 64;
+    constexpr int SWZ = CPR >= 16 ? 15 : 7;        // rows 256 bytes long all start at one bank: their 16 chunks are permuted as a whole
     static_assert(!SHORT || KS == 64, "the short load path is written for steps of 64");
     __shared__ __attribute__((aligned(16))) bf16_t As[BM * LDS];
     __shared__ __attribute__((aligned(16))) bf16_t Bs[BN * LDS];
@@ -116,12 +117,12 @@ gemm_mfma_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __
     auto stage = [&]() {
 #pragma unroll
         for (int i = 0; i < LA; i++) {
-            const int c = tid + i * 256, row = c / CPR, kc = ((c % CPR) ^ (row & 7)) * 8;  // chunk j of a row sits at j ^ (row & 7)
+            const int c = tid + i * 256, row = c / CPR, kc = ((c % CPR) ^ (row & SWZ)) * 8;  // chunk j of a row sits at j ^ (row & SWZ)
             *reinterpret_cast<bf16x8*>(As + row * LDS + kc) = ra[i];
         }
 #pragma unroll
         for (int i = 0; i < LB; i++) {
-            const int c = tid + i * 256, row = c / CPR, kc = ((c % CPR) ^ (row & 7)) * 8;
+            const int c = tid + i * 256, row = c / CPR, kc = ((c % CPR) ^ (row & SWZ)) * 8;
             *reinterpret_cast<bf16x8*>(Bs + row * LDS + kc) = rb[i];
         }
     };
@@ -141,7 +142,7 @@ gemm_mfma_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __
 #pragma unroll
         for (int ks = 0; ks < BK; ks += 32) {
             Frag a[TM], b[TN];
-            const int kc = (((ks >> 3) + g) ^ (r & 7)) * 8;
+            const int kc = (((ks >> 3) + g) ^ (r & SWZ)) * 8;
 #pragma unroll
             for (int i = 0; i < TM; i++) a[i].u = *reinterpret_cast<const uint4*>(As + (wm * 16 * TM + i * 16 + r) * LDS + kc);
 #pragma unroll
