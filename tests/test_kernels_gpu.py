@@ -67,7 +67,7 @@ def test_add_rms_norm(ops, dt, post, nxt, m, d):
 
 
 @pytest.mark.parametrize("m,n,k", [(8, 2304, 2048), (3, 600, 9216), (64, 2304, 4096), (700, 2304, 2048), (300, 520, 4104),
-                                   (2048, 2304, 4096)])
+                                   (2048, 2304, 4096), (1, 2304, 9216), (2, 601, 14336)])
 def test_deferred_product_into_add_rms_norm(ops, m, n, k):
     """A product left in K slices and added by add_rms_norm equals the product, then the norm."""
     from trapetum_amd.kernels.ops import SplitRows
@@ -101,11 +101,17 @@ LINEAR_SHAPES += [(65, 100, 64), (300, 257, 576), (1000, 520, 192), (513, 2304, 
 LINEAR_SHAPES += [(300, 44177, 64), (40, 70001, 72)]
 
 
-@pytest.mark.parametrize("algo", [1, 2, 3, 6, 7])
+# one and two rows, for the kernel that takes no more: widths of one to ten chunks a lane, an odd number of rows of W
+LINEAR_SHAPES += [(1, 77, 8), (2, 301, 1000), (2, 130, 1536), (1, 257, 3584), (2, 99, 4608), (1, 64, 5120)]
+
+
+@pytest.mark.parametrize("algo", [1, 2, 3, 4, 6, 7])
 @pytest.mark.parametrize("m,n,k", LINEAR_SHAPES)
 def test_linear_bf16(ops, algo, m, n, k):
     if algo == 2 and m > 64:
         pytest.skip("the skinny kernel takes at most 64 rows")
+    if algo == 4 and (m > 2 or k > 5120):
+        pytest.skip("the multiply-add kernel takes at most 2 rows and, unsliced, a K of 5120")
     x, w = randn(m, k, dtype=torch.bfloat16, seed=7), randn(n, k, dtype=torch.bfloat16, seed=8, scale=0.05)
     ops.force_linear = algo
     try:
@@ -131,13 +137,15 @@ def test_linear_f32(ops, m, n, k):
     assert torch.equal(alone[0], got[m - 1])
 
 
-@pytest.mark.parametrize("algo", [1, 2, 3, 6])
+@pytest.mark.parametrize("algo", [1, 2, 3, 4, 6])
 @pytest.mark.parametrize("dt", ["bf16", "f32"])
 @pytest.mark.parametrize("m,inter,k", [(1, 16, 16), (4, 200, 88), (40, 320, 96), (9, 1000, 2304), (150, 72, 136),
-                                       (150, 72, 128), (700, 1000, 320), (130, 36010, 64)])
+                                       (150, 72, 128), (700, 1000, 320), (130, 36010, 64), (2, 1000, 2304), (1, 75, 4608)])
 def test_gated_linear(ops, algo, dt, m, inter, k):
     if dt == "f32" and algo != 1:
         pytest.skip("float32 runs on the plain kernel only")
+    if algo == 4 and m > 2:
+        pytest.skip("the multiply-add kernel takes at most 2 rows")
     if algo == 2 and m > 64:
         pytest.skip("the skinny kernel takes at most 64 rows")
     wg, wu = randn(inter, k, dtype=DT[dt], seed=11, scale=0.2), randn(inter, k, dtype=DT[dt], seed=12, scale=0.2)

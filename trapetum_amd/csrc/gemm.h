@@ -13,7 +13,7 @@ struct GemmArgs {
     int units;              // gated: columns of the output (the feed-forward width)
     void* workspace; size_t workspace_bytes;
     int defer;              // split products: leave the K slices in the workspace [slices, M, N] for the consumer to add
-    int algo;               // the caller's choice of kernel (0: none); 6 asks the tiled kernel for its wide tile
+    int algo;               // the caller's choice of kernel (0: none; see tp_linear)
     hipStream_t stream;
 };
 
@@ -23,6 +23,10 @@ int gemm_simple_launch(const GemmArgs& a);
 bool gemm_skinny_supports(const GemmArgs& a);
 size_t gemm_skinny_workspace(const GemmArgs& a);
 int gemm_skinny_launch(const GemmArgs& a);
+// bf16 by plain multiply-adds for one or two rows: X in registers, W streamed in contiguous kilobytes
+bool gemv_supports(const GemmArgs& a);
+size_t gemv_workspace(const GemmArgs& a);
+int gemv_launch(const GemmArgs& a);
 bool gemm_mfma_supports(const GemmArgs& a);
 int gemm_mfma_splits(const GemmArgs& a);
 int gemm_mfma_launch(const GemmArgs& a);

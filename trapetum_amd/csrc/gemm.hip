@@ -103,9 +103,11 @@ static int check_args(const GemmArgs& a) {
     return 0;
 }
 
-// algo: 0 = choose, 1 = plain, 2 = skinny matrix-core, 3 = tiled matrix-core (6: with its wide tile, 7: with its 128 x 96 tile)
+// algo: 0 = choose, 1 = plain, 2 = skinny matrix-core, 3 = tiled matrix-core (6: with its wide tile, 7: with its 128 x 96 tile),
+// 4 = multiply-adds for one or two rows
 static int pick(const GemmArgs& a, int algo) {
     if (algo == 1) return 1;
+    if (algo == 4) return gemv_supports(a) ? 4 : -4;
     if (algo == 2) return gemm_skinny_supports(a) ? 2 : -2;
     if (algo == 3 || algo == 6 || algo == 7) return gemm_mfma_supports(a) ? 3 : -3;
     // Up to 64 rows both matrix-core kernels stream W once; which is faster was measured on MI355X at the 2B shapes
@@ -115,6 +117,7 @@ static int pick(const GemmArgs& a, int algo) {
     //   qkv     N 4096  K 2304      8 rows  8.0 /  7.1   32 rows 11.7 /  7.5   64 rows 13.5 /  8.5   (K slices)
     //   o       N 2304  K 2048      8 rows  5.2 /  5.5   32 rows  7.7 /  6.0   64 rows 13.3 /  6.7   (K slices)
     //   gate/up N 18432 K 2304      8 rows 26.9 / 24.2   32 rows 40.7 / 24.7   64 rows 48.5 / 26.5   (no slices: gated)
+    if (gemv_supports(a)) return 4;          // one or two rows: 2B gate/up 16.8 against 22.6 us on the skinny kernel
     if (gemm_mfma_supports(a)) {
         const bool sliced = a.defer && a.epilogue == TP_EPI_NONE;
         // (up to 16 rows the tiled kernel's lead on qkv and down is lost again in their consumers, which then add
@@ -138,6 +141,7 @@ extern "C" long tp_linear_workspace_bytes(int in_dtype, int out_dtype, int M, in
     GemmArgs a{nullptr, nullptr, nullptr, in_dtype, out_dtype, M, N, K, epilogue, 1.f, units, nullptr, 0, defer, algo, nullptr};
     const int p = pick(a, algo);
     if (p == 2) return (long)gemm_skinny_workspace(a);
+    if (p == 4) return (long)gemv_workspace(a);
     if (p == 3) { const int s = gemm_mfma_splits(a); return s > 1 ? (long)s * M * N * 4 : 0; }
     if (p == 1 && epilogue == TP_EPI_GATED) return (long)M * N * 4;
     return 0;
@@ -152,6 +156,7 @@ extern "C" int tp_linear(const void* x, const void* w, void* y, int in_dtype, in
     const int p = pick(a, algo);
     TP_REQUIRE(p > 0, "linear: the requested kernel (%d) does not take M=%d N=%d K=%d dtype %d", algo, M, N, K, in_dtype);
     if (p == 2) return gemm_skinny_launch(a);
+    if (p == 4) return gemv_launch(a);
     if (p == 3) return gemm_mfma_launch(a);
     return gemm_simple_launch(a);
 }
