@@ -105,9 +105,11 @@ LINEAR_SHAPES += [(300, 44177, 64), (40, 70001, 72)]
 LINEAR_SHAPES += [(1, 77, 8), (2, 301, 1000), (2, 130, 1536), (1, 257, 3584), (2, 99, 4608), (1, 64, 5120)]
 
 
-@pytest.mark.parametrize("algo", [1, 2, 3, 4, 6, 7])
+@pytest.mark.parametrize("algo", [1, 2, 3, 4, 6, 7, 8])
 @pytest.mark.parametrize("m,n,k", LINEAR_SHAPES)
 def test_linear_bf16(ops, algo, m, n, k):
+    if algo == 8 and k % 64:
+        pytest.skip("the loop that loads straight into LDS takes whole k steps of 64")
     if algo == 2 and m > 64:
         pytest.skip("the skinny kernel takes at most 64 rows")
     if algo == 4 and (m > 2 or k > 5120):
@@ -137,7 +139,7 @@ def test_linear_f32(ops, m, n, k):
     assert torch.equal(alone[0], got[m - 1])
 
 
-@pytest.mark.parametrize("algo", [1, 2, 3, 4, 6])
+@pytest.mark.parametrize("algo", [1, 2, 3, 4, 6, 8])
 @pytest.mark.parametrize("dt", ["bf16", "f32"])
 @pytest.mark.parametrize("m,inter,k", [(1, 16, 16), (4, 200, 88), (40, 320, 96), (9, 1000, 2304), (150, 72, 136),
                                        (150, 72, 128), (700, 1000, 320), (130, 36010, 64), (2, 1000, 2304), (1, 75, 4608)])
@@ -148,6 +150,8 @@ def test_gated_linear(ops, algo, dt, m, inter, k):
         pytest.skip("the multiply-add kernel takes at most 2 rows")
     if algo == 2 and m > 64:
         pytest.skip("the skinny kernel takes at most 64 rows")
+    if algo == 8 and k % 64:
+        pytest.skip("the loop that loads straight into LDS takes whole k steps of 64")
     wg, wu = randn(inter, k, dtype=DT[dt], seed=11, scale=0.2), randn(inter, k, dtype=DT[dt], seed=12, scale=0.2)
     x = randn(m, k, dtype=DT[dt], seed=13)
     packed = ops.pack_gate_up(wg, wu)

@@ -31,6 +31,51 @@ __device__ __forceinline__ unsigned in_register(unsigned v) {
 }
 }
 
+// A wave's accumulators to Y.  The lane holds Y[m = .. + r][n = .. + g*4 + v], v = 0..3: four neighbours of a row go
+// out in one store where the row length allows the alignment.
+template <int EPI, int TM, int TN>
+__device__ __forceinline__ void store_tile(const f32x4 (&acc)[TM][TN], void* __restrict__ Y, int M, int N, int m0, int n0,
+                                           int wm, int wn, int r, int g, int out_dtype, float cap, int units) {
+    const int width = EPI == TP_EPI_GATED ? units : N;
+    const bool wide = (width & 3) == 0;
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+        const int m = m0 + wm * 16 * TM + i * 16 + r;
+        if (m >= M) continue;
+#pragma unroll
+        for (int j = 0; j < TN; j += (EPI == TP_EPI_GATED ? 2 : 1)) {
+            float o[4];
+            int col;                                            // first of the four columns of Y (units if gated)
+            if (EPI == TP_EPI_GATED) {
+                col = ((n0 + wn * 16 * TN + j * 16) >> 1) + g * 4;
+#pragma unroll
+                for (int v = 0; v < 4; v++) o[v] = gelu_tanh_fast(acc[i][j][v]) * acc[i][j + 1 < TN ? j + 1 : j][v];
+            } else {
+                col = n0 + wn * 16 * TN + j * 16 + g * 4;
+#pragma unroll
+                for (int v = 0; v < 4; v++) o[v] = EPI == TP_EPI_SOFTCAP ? softcap_f(acc[i][j][v], cap) : acc[i][j][v];
+            }
+            if (col >= width) continue;
+            const size_t at = (size_t)m * width + col;
+            if (wide) {                                         // width % 4 == 0 and col % 4 == 0: all four are inside
+                if (out_dtype == TP_F32) *reinterpret_cast<f32x4*>((float*)Y + at) = (f32x4){o[0], o[1], o[2], o[3]};
+                else {
+                    ushort4 pk;
+                    pk.x = f32_to_bf16(o[0]); pk.y = f32_to_bf16(o[1]); pk.z = f32_to_bf16(o[2]); pk.w = f32_to_bf16(o[3]);
+                    *reinterpret_cast<ushort4*>((bf16_t*)Y + at) = pk;
+                }
+            } else {
+#pragma unroll
+                for (int v = 0; v < 4; v++) {
+                    if (col + v >= width) break;
+                    if (out_dtype == TP_F32) ((float*)Y)[at + v] = o[v];
+                    else ((bf16_t*)Y)[at + v] = f32_to_bf16(o[v]);
+                }
+            }
+        }
+    }
+}
+
 // TM x TN: the 16 x 16 tiles of a wave; the block's 2 x 2 waves cover BM = 32 TM rows of X and BN = 32 TN rows of W
 // SHORT: whole tiles load their k steps by the short path described below
 // KS: elements of a k step (64, or 128 for the 64 x 64 tiles, which stream W and are bound by the bytes a block has
@@ -155,49 +200,94 @@ gemm_mfma_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __
         }
     }
 
-    // lane holds Y[m = .. + r][n = .. + g*4 + v], v = 0..3: four neighbours of a row go out in one store where the
-    // row length allows the alignment
-    const int width = EPI == TP_EPI_GATED ? units : N;
-    const bool wide = (width & 3) == 0;
+    store_tile<EPI, TM, TN>(acc, Y, M, N, m0, n0, wm, wn, r, g, out_dtype, cap, units);
+}
+
+// 128 x 128 tiles for grids of at most two blocks a CU (narrow products of a prefill: the attention's projections).
+// There the loop above leaves the matrix cores waiting: a block's loads are one k step ahead and few blocks stand in.
+// This loop keeps two LDS buffers and fills the other one by loads that go from global memory straight into LDS
+// (global_load_lds_dwordx4: no staging registers, no LDS write instructions), issued after the step's fragment
+// reads and before its products; one barrier a step.  A lane's place in LDS is fixed by its lane number (16 bytes on
+// from its neighbour's), so the swizzle is applied to the global side: the lane whose place is (row, j) fetches
+// chunk j ^ (row & 7) of that row.  Rows past the edge of Y fetch the last row (their products are never stored); K must be a
+// multiple of 64.  64 KB of LDS: two blocks a CU, so a grid runs in rounds of 512 blocks and one that fills its
+// rounds badly stays with the loop above (three blocks a CU).  Measured at the 2B shapes: qkv at 2,048 rows 55 -> 43 us
+// (512 tiles), at 4,096 rows 90 -> 83 us (1,024 tiles); o at 4,096 rows 50 -> 66 us (576 tiles: not chosen).
+template <int EPI>
+__global__ void __launch_bounds__(256, 2)
+gemm_mfma_direct_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __restrict__ Y,
+                   int M, int N, int K, int m_tiles, int out_dtype, float cap, int units, int k_per_split) {
+    constexpr int TM = 4, TN = 4, BM = 128, BN = 128, LDS = BK, BUF = (BM + BN) * LDS;
+    extern __shared__ __attribute__((aligned(16))) bf16_t smem[];          // [2][BUF]
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 15, g = lane >> 4;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int m0 = (blockIdx.x % m_tiles) * BM, n0 = (blockIdx.x / m_tiles) * BN;
+    const int k_begin = blockIdx.y * k_per_split;
+    const int k_end = min(K, k_begin + k_per_split);
+    if (gridDim.y > 1) Y = (float*)Y + (size_t)blockIdx.y * M * N;
+
+    // load i of a thread: row (tid >> 3) + 32 i of the tile, the chunk that belongs at the lane's place
+    const int srow = tid >> 3, chunk = (lane & 7) ^ (srow & 7);
+    unsigned xo[TM], wo[TN];
 #pragma unroll
-    for (int i = 0; i < TM; i++) {
-        const int m = m0 + wm * 16 * TM + i * 16 + r;
-        if (m >= M) continue;
+    for (int i = 0; i < TM; i++) xo[i] = (unsigned)min(m0 + srow + 32 * i, M - 1) * (unsigned)K * 2u + chunk * 16u;
 #pragma unroll
-        for (int j = 0; j < TN; j += (EPI == TP_EPI_GATED ? 2 : 1)) {
-            float o[4];
-            int col;                                            // first of the four columns of Y (units if gated)
-            if (EPI == TP_EPI_GATED) {
-                col = ((n0 + wn * 16 * TN + j * 16) >> 1) + g * 4;
+    for (int i = 0; i < TN; i++) wo[i] = (unsigned)min(n0 + srow + 32 * i, N - 1) * (unsigned)K * 2u + chunk * 16u;
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    auto fill = [&](int k0, int buf) {
+        bf16_t* As = smem + buf * BUF + wave_u * 8 * LDS;                  // the wave's 8 rows of every group of 32
+        bf16_t* Bs = As + BM * LDS;
+        const char* xb = reinterpret_cast<const char*>(X) + (size_t)k0 * 2;
+        const char* wb = reinterpret_cast<const char*>(W) + (size_t)k0 * 2;
 #pragma unroll
-                for (int v = 0; v < 4; v++) o[v] = gelu_tanh_fast(acc[i][j][v]) * acc[i][j + 1 < TN ? j + 1 : j][v];
-            } else {
-                col = n0 + wn * 16 * TN + j * 16 + g * 4;
+        for (int i = 0; i < TM; i++)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(xb + xo[i]),
+                                             (__attribute__((address_space(3))) void*)(As + 32 * i * LDS), 16, 0, 0);
 #pragma unroll
-                for (int v = 0; v < 4; v++) o[v] = EPI == TP_EPI_SOFTCAP ? softcap_f(acc[i][j][v], cap) : acc[i][j][v];
-            }
-            if (col >= width) continue;
-            const size_t at = (size_t)m * width + col;
-            if (wide) {                                         // width % 4 == 0 and col % 4 == 0: all four are inside
-                if (out_dtype == TP_F32) *reinterpret_cast<f32x4*>((float*)Y + at) = (f32x4){o[0], o[1], o[2], o[3]};
-                else {
-                    ushort4 pk;
-                    pk.x = f32_to_bf16(o[0]); pk.y = f32_to_bf16(o[1]); pk.z = f32_to_bf16(o[2]); pk.w = f32_to_bf16(o[3]);
-                    *reinterpret_cast<ushort4*>((bf16_t*)Y + at) = pk;
-                }
-            } else {
+        for (int i = 0; i < TN; i++)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(wb + wo[i]),
+                                             (__attribute__((address_space(3))) void*)(Bs + 32 * i * LDS), 16, 0, 0);
+    };
+    f32x4 acc[TM][TN];
 #pragma unroll
-                for (int v = 0; v < 4; v++) {
-                    if (col + v >= width) break;
-                    if (out_dtype == TP_F32) ((float*)Y)[at + v] = o[v];
-                    else ((bf16_t*)Y)[at + v] = f32_to_bf16(o[v]);
-                }
-            }
-        }
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    auto frags = [&](const bf16_t* As, const bf16_t* Bs, int ks, Frag (&a)[TM], Frag (&b)[TN]) {
+        const int kc = (((ks >> 3) + g) ^ (r & 7)) * 8;
+#pragma unroll
+        for (int i = 0; i < TM; i++) a[i].u = *reinterpret_cast<const uint4*>(As + (wm * 16 * TM + i * 16 + r) * LDS + kc);
+#pragma unroll
+        for (int j = 0; j < TN; j++) b[j].u = *reinterpret_cast<const uint4*>(Bs + (wn * 16 * TN + j * 16 + r) * LDS + kc);
+    };
+    auto mma = [&](Frag (&a)[TM], Frag (&b)[TN]) {
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b[j].v, a[i].v, acc[i][j], 0, 0, 0);
+    };
+    fill(k_begin, 0);
+    __builtin_amdgcn_s_waitcnt(0);                   // every counter at zero: the loads have reached LDS
+    __syncthreads();
+    int cur = 0;
+    for (int k0 = k_begin; k0 < k_end; k0 += BK) {
+        const bf16_t* As = smem + cur * BUF, * Bs = As + BM * LDS;
+        Frag a0[TM], b0[TN], a1[TM], b1[TN];
+        frags(As, Bs, 0, a0, b0);
+        frags(As, Bs, 32, a1, b1);
+        if (k0 + BK < k_end) fill(k0 + BK, cur ^ 1);   // the other buffer was last read a barrier ago
+        mma(a0, b0);
+        mma(a1, b1);
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+        cur ^= 1;
     }
+    store_tile<EPI, TM, TN>(acc, Y, M, N, m0, n0, wm, wn, r, g, out_dtype, cap, units);
 }
 
 bool gemm_mfma_supports(const GemmArgs& a) {
+    if (a.algo == 8) return a.in_dtype == TP_BF16 && a.K % BK == 0 && (long)(a.M > a.N ? a.M : a.N) * a.K * 2 < (1L << 32);
     return a.in_dtype == TP_BF16 && a.K % 8 == 0;
 }
 
@@ -207,7 +297,7 @@ bool gemm_mfma_supports(const GemmArgs& a) {
 // else 128 x 128 or 128 x 96 (three blocks a CU).  Measured on the 2B gate/up product: 930 against 790 TFLOP/s at
 // 8192 rows, 700 against 790 at 2048; at 64 rows 35 us with 64 x 64 tiles against 45 us with 128 x 128.
 struct Tile { int tm, tn; };
-struct Plan { Tile tile; int splits; };
+struct Plan { Tile tile; int splits; bool direct = false; };
 
 // K slices of a product of few rows, which is bound by reading W and wants every CU streaming
 static int small_tile_splits(const GemmArgs& a, long blocks) {
@@ -234,7 +324,19 @@ static Plan mid_tile_plan(const GemmArgs& a, bool may_slice) {
             if (s > 1 && a.K / s < 512) break;
             const double k_steps = (double)tp_cdiv(tp_cdiv(a.K, s), BK);
             const double cost = (double)tp_cdiv(tiles * s, 256) * k_steps * step_us * (tn == 3 ? 0.8 : 1.0) + (s - 1) * slice_us;
-            if (cost < best_cost * 0.97) { best_cost = cost; best = {{4, tn}, s}; }      // a tie stays with the earlier, plainer plan
+            if (cost < best_cost * 0.97) { best_cost = cost; best = {{4, tn}, s, false}; }      // a tie stays with the earlier, plainer plan
+        }
+    }
+    // the loop with loads straight into LDS: 128 x 128 tiles, two blocks a CU (64 KB of LDS each), so rounds of 512
+    // blocks; a k step takes 1.15 us whether a CU holds one block or two (at 2,048 rows: o 288 blocks 35 us, qkv 512
+    // blocks 43 us, down 288 blocks 134 us; at 4,096 rows: qkv 1,024 blocks 83 us, o 576 blocks 66 us)
+    if (a.K % BK == 0 && a.algo != 7 && (long)(a.M > a.N ? a.M : a.N) * a.K * 2 < (1L << 32)) {    // (32-bit row offsets)
+        const long tiles = (long)tp_cdiv(a.M, 128) * tp_cdiv(a.N, 128);
+        for (int s = 1; s <= (may_slice ? 4 : 1); s++) {
+            if (s > 1 && a.K / s < 512) break;
+            const double k_steps = (double)tp_cdiv(tp_cdiv(a.K, s), BK);
+            const double cost = (double)tp_cdiv(tiles * s, 512) * k_steps * 1.15 + 2.0 + (s - 1) * slice_us;
+            if (cost < best_cost * 0.97) { best_cost = cost; best = {{4, 4}, s, true}; }
         }
     }
     return best;
@@ -243,6 +345,7 @@ static Plan mid_tile_plan(const GemmArgs& a, bool may_slice) {
 static Plan plan_of(const GemmArgs& a) {
     const bool may_slice = a.defer && a.epilogue == TP_EPI_NONE && a.algo != 6 && a.algo != 7;
     if (a.algo == 6) return {{4, 8}, 1};
+    if (a.algo == 8) return {{4, 4}, 1, true};
     if (a.algo == 7) return {{4, a.epilogue == TP_EPI_GATED ? 4 : 3}, 1};
     // the logits of 64 rows: 250 us with 128 x 128, 275 with 64 x 64; up to 256 rows of a narrow product: 128 x 128
     // tiles would leave most CUs idle (down at 128 rows: 44 us on 72 blocks, against 15 us at 64 rows on 576 blocks
@@ -270,6 +373,17 @@ static void mfma_launch(const GemmArgs& a, void* y, int out_dtype, int splits, i
 }
 
 template <int EPI>
+static int mfma_launch_direct(const GemmArgs& a, void* y, int out_dtype, int splits, int kps) {
+    static const hipError_t attr = hipFuncSetAttribute((const void*)gemm_mfma_direct_k<EPI>, hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
+    TP_REQUIRE(attr == hipSuccess, "tiled product: 64 KB of LDS refused (%s)", hipGetErrorString(attr));
+    const int m_tiles = tp_cdiv(a.M, 128), n_tiles = tp_cdiv(a.N, 128);
+    dim3 grid((unsigned)(m_tiles * n_tiles), splits);
+    gemm_mfma_direct_k<EPI><<<grid, 256, 65536, a.stream>>>((const bf16_t*)a.x, (const bf16_t*)a.w, y, a.M, a.N, a.K, m_tiles,
+                                                             out_dtype, a.cap, a.units, kps);
+    return 0;
+}
+
+template <int EPI>
 static void mfma_launch_tile(const GemmArgs& a, Tile t, void* y, int out_dtype, int splits, int kps) {
     if (t.tm == 2) mfma_launch<EPI, 2, 2, SMALL_KS>(a, y, out_dtype, splits, kps);
     else if (t.tn == 8) mfma_launch<EPI, 4, 8>(a, y, out_dtype, splits, kps);
@@ -291,8 +405,16 @@ int gemm_mfma_launch(const GemmArgs& a) {
         TP_REQUIRE(a.workspace && a.workspace_bytes >= need, "tiled product: workspace of %zu bytes, %zu needed", a.workspace_bytes, need);
         const int kstep = t.tm == 2 ? SMALL_KS : BK;
         const int kps = tp_cdiv(tp_cdiv(a.K, splits), kstep) * kstep;
-        mfma_launch_tile<TP_EPI_NONE>(a, t, a.workspace, TP_F32, tp_cdiv(a.K, kps), kps);
+        if (plan.direct) { if (int rc = mfma_launch_direct<TP_EPI_NONE>(a, a.workspace, TP_F32, tp_cdiv(a.K, kps), kps)) return rc; }
+        else mfma_launch_tile<TP_EPI_NONE>(a, t, a.workspace, TP_F32, tp_cdiv(a.K, kps), kps);
         return tp_check_launch("linear (tiled kernel, K slices)");
+    }
+    if (plan.direct) {
+        int rc;
+        if (a.epilogue == TP_EPI_GATED) rc = mfma_launch_direct<TP_EPI_GATED>(a, a.y, a.out_dtype, 1, a.K);
+        else if (a.epilogue == TP_EPI_SOFTCAP) rc = mfma_launch_direct<TP_EPI_SOFTCAP>(a, a.y, a.out_dtype, 1, a.K);
+        else rc = mfma_launch_direct<TP_EPI_NONE>(a, a.y, a.out_dtype, 1, a.K);
+        return rc ? rc : tp_check_launch("linear (tiled kernel, loads into LDS)");
     }
     if (a.epilogue == TP_EPI_GATED) mfma_launch_tile<TP_EPI_GATED>(a, t, a.y, a.out_dtype, 1, a.K);
     else if (a.epilogue == TP_EPI_SOFTCAP) mfma_launch_tile<TP_EPI_SOFTCAP>(a, t, a.y, a.out_dtype, 1, a.K);
