@@ -105,10 +105,10 @@ LINEAR_SHAPES += [(300, 44177, 64), (40, 70001, 72)]
 LINEAR_SHAPES += [(1, 77, 8), (2, 301, 1000), (2, 130, 1536), (1, 257, 3584), (2, 99, 4608), (1, 64, 5120)]
 
 
-@pytest.mark.parametrize("algo", [1, 2, 3, 4, 6, 7, 8])
+@pytest.mark.parametrize("algo", [1, 2, 3, 4, 6, 7, 8, 9])
 @pytest.mark.parametrize("m,n,k", LINEAR_SHAPES)
 def test_linear_bf16(ops, algo, m, n, k):
-    if algo == 8 and k % 64:
+    if algo in (8, 9) and k % 64:
         pytest.skip("the loop that loads straight into LDS takes whole k steps of 64")
     if algo == 2 and m > 64:
         pytest.skip("the skinny kernel takes at most 64 rows")
@@ -150,7 +150,7 @@ def test_gated_linear(ops, algo, dt, m, inter, k):
         pytest.skip("the multiply-add kernel takes at most 2 rows")
     if algo == 2 and m > 64:
         pytest.skip("the skinny kernel takes at most 64 rows")
-    if algo == 8 and k % 64:
+    if algo in (8, 9) and k % 64:
         pytest.skip("the loop that loads straight into LDS takes whole k steps of 64")
     wg, wu = randn(inter, k, dtype=DT[dt], seed=11, scale=0.2), randn(inter, k, dtype=DT[dt], seed=12, scale=0.2)
     x = randn(m, k, dtype=DT[dt], seed=13)

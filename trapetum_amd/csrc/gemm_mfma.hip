@@ -203,25 +203,38 @@ gemm_mfma_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __
     store_tile<EPI, TM, TN>(acc, Y, M, N, m0, n0, wm, wn, r, g, out_dtype, cap, units);
 }
 
-// 128 x 128 tiles for grids of at most two blocks a CU (narrow products of a prefill: the attention's projections).
-// There the loop above leaves the matrix cores waiting: a block's loads are one k step ahead and few blocks stand in.
-// This loop keeps two LDS buffers and fills the other one by loads that go from global memory straight into LDS
-// (global_load_lds_dwordx4: no staging registers, no LDS write instructions), issued after the step's fragment
-// reads and before its products; one barrier a step.  A lane's place in LDS is fixed by its lane number (16 bytes on
-// from its neighbour's), so the swizzle is applied to the global side: the lane whose place is (row, j) fetches
-// chunk j ^ (row & 7) of that row.  Rows past the edge of Y fetch the last row (their products are never stored); K must be a
-// multiple of 64.  64 KB of LDS: two blocks a CU, so a grid runs in rounds of 512 blocks and one that fills its
-// rounds badly stays with the loop above (three blocks a CU).  Measured at the 2B shapes: qkv at 2,048 rows 55 -> 43 us
-// (512 tiles), at 4,096 rows 90 -> 83 us (1,024 tiles); o at 4,096 rows 50 -> 66 us (576 tiles: not chosen).
-template <int EPI>
+// The loop of the large tiles (128 x 128 and 128 x 96) when K is a multiple of 64: the k step's tile comes from
+// global memory straight into LDS (global_load_lds_dwordx4: no staging registers, no LDS write instructions).  One LDS
+// buffer, as above, so that three blocks fit a CU: a step reads all its fragments into registers, a barrier, then the
+// loads of the next step are issued into the same buffer and fly while the step's 32 matrix instructions run; a
+// second barrier when they have landed.  A lane's place in LDS is fixed by its lane number (16 bytes on from its
+// neighbour's), so the swizzle is applied on the global side: the lane whose place is (row, j) fetches chunk
+// j ^ (row & 7) of that row.  Rows past the edge of Y fetch the last row (their products are never stored).
+// Measured at the 2B shapes against the register-staged loop: gate/up at 2,048 rows 185 -> 155 us (1.1 PFLOP/s), at
+// 8,192 rows 660 (128 x 256 tiles) -> 632 us; qkv at 2,048 rows 52 -> 42 us; down, unsliced, 133 -> 125 us.
+// (Two LDS buffers with one barrier a step were no faster and leave two blocks a CU.)
+template <int EPI, int TN>
 __global__ void __launch_bounds__(256, 2)
 gemm_mfma_direct_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __restrict__ Y,
-                   int M, int N, int K, int m_tiles, int out_dtype, float cap, int units, int k_per_split) {
-    constexpr int TM = 4, TN = 4, BM = 128, BN = 128, LDS = BK, BUF = (BM + BN) * LDS;
-    extern __shared__ __attribute__((aligned(16))) bf16_t smem[];          // [2][BUF]
+                   int M, int N, int K, int m_tiles, int out_dtype, float cap, int units, int k_per_split, int xcd_panels) {
+    constexpr int TM = 4, BM = 128, BN = 32 * TN, LDS = BK;
+    __shared__ __attribute__((aligned(16))) bf16_t As[BM * LDS];
+    __shared__ __attribute__((aligned(16))) bf16_t Bs[BN * LDS];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 15, g = lane >> 4;
     const int wm = wave >> 1, wn = wave & 1;
-    const int m0 = (blockIdx.x % m_tiles) * BM, n0 = (blockIdx.x / m_tiles) * BN;
+    int vb = blockIdx.x, mt, nt;                     // the order of the tiles: as in gemm_mfma_k
+    if (xcd_panels) {
+        const int total = gridDim.x, base = total >> 3, rem = total & 7, xcd = vb & 7;
+        vb = xcd * base + min(xcd, rem) + (vb >> 3);
+        const int n_tiles = total / m_tiles, per_panel = 4 * m_tiles, p = vb / per_panel, q = vb - p * per_panel;
+        const int width = min(4, n_tiles - p * 4);
+        nt = p * 4 + q % width;
+        mt = q / width;
+    } else {
+        mt = vb % m_tiles;
+        nt = vb / m_tiles;
+    }
+    const int m0 = mt * BM, n0 = nt * BN;
     const int k_begin = blockIdx.y * k_per_split;
     const int k_end = min(K, k_begin + k_per_split);
     if (gridDim.y > 1) Y = (float*)Y + (size_t)blockIdx.y * M * N;
@@ -234,26 +247,26 @@ gemm_mfma_direct_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, v
 #pragma unroll
     for (int i = 0; i < TN; i++) wo[i] = (unsigned)min(n0 + srow + 32 * i, N - 1) * (unsigned)K * 2u + chunk * 16u;
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
-    auto fill = [&](int k0, int buf) {
-        bf16_t* As = smem + buf * BUF + wave_u * 8 * LDS;                  // the wave's 8 rows of every group of 32
-        bf16_t* Bs = As + BM * LDS;
+    bf16_t* const a_dst = As + wave_u * 8 * LDS;     // the wave's 8 rows of every group of 32
+    bf16_t* const b_dst = Bs + wave_u * 8 * LDS;
+    auto fill = [&](int k0) {
         const char* xb = reinterpret_cast<const char*>(X) + (size_t)k0 * 2;
         const char* wb = reinterpret_cast<const char*>(W) + (size_t)k0 * 2;
 #pragma unroll
         for (int i = 0; i < TM; i++)
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(xb + xo[i]),
-                                             (__attribute__((address_space(3))) void*)(As + 32 * i * LDS), 16, 0, 0);
+                                             (__attribute__((address_space(3))) void*)(a_dst + 32 * i * LDS), 16, 0, 0);
 #pragma unroll
         for (int i = 0; i < TN; i++)
             __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(wb + wo[i]),
-                                             (__attribute__((address_space(3))) void*)(Bs + 32 * i * LDS), 16, 0, 0);
+                                             (__attribute__((address_space(3))) void*)(b_dst + 32 * i * LDS), 16, 0, 0);
     };
     f32x4 acc[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; i++)
 #pragma unroll
         for (int j = 0; j < TN; j++) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    auto frags = [&](const bf16_t* As, const bf16_t* Bs, int ks, Frag (&a)[TM], Frag (&b)[TN]) {
+    auto frags = [&](int ks, Frag (&a)[TM], Frag (&b)[TN]) {
         const int kc = (((ks >> 3) + g) ^ (r & 7)) * 8;
 #pragma unroll
         for (int i = 0; i < TM; i++) a[i].u = *reinterpret_cast<const uint4*>(As + (wm * 16 * TM + i * 16 + r) * LDS + kc);
@@ -267,35 +280,34 @@ gemm_mfma_direct_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, v
             for (int j = 0; j < TN; j++)
                 acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b[j].v, a[i].v, acc[i][j], 0, 0, 0);
     };
-    fill(k_begin, 0);
+    fill(k_begin);
     __builtin_amdgcn_s_waitcnt(0);                   // every counter at zero: the loads have reached LDS
     __syncthreads();
-    int cur = 0;
     for (int k0 = k_begin; k0 < k_end; k0 += BK) {
-        const bf16_t* As = smem + cur * BUF, * Bs = As + BM * LDS;
         Frag a0[TM], b0[TN], a1[TM], b1[TN];
-        frags(As, Bs, 0, a0, b0);
-        frags(As, Bs, 32, a1, b1);
-        if (k0 + BK < k_end) fill(k0 + BK, cur ^ 1);   // the other buffer was last read a barrier ago
+        frags(0, a0, b0);
+        frags(32, a1, b1);
+        __builtin_amdgcn_s_waitcnt(0);               // the fragments are in registers ...
+        __syncthreads();                             // ... everyone's: the buffer may be refilled
+        if (k0 + BK < k_end) fill(k0 + BK);
         mma(a0, b0);
         mma(a1, b1);
         __builtin_amdgcn_s_waitcnt(0);
         __syncthreads();
-        cur ^= 1;
     }
     store_tile<EPI, TM, TN>(acc, Y, M, N, m0, n0, wm, wn, r, g, out_dtype, cap, units);
 }
 
 bool gemm_mfma_supports(const GemmArgs& a) {
-    if (a.algo == 8) return a.in_dtype == TP_BF16 && a.K % BK == 0 && (long)(a.M > a.N ? a.M : a.N) * a.K * 2 < (1L << 32);
+    if (a.algo == 8 || a.algo == 9) return a.in_dtype == TP_BF16 && a.K % BK == 0 && (long)(a.M > a.N ? a.M : a.N) * a.K * 2 < (1L << 32);
     return a.in_dtype == TP_BF16 && a.K % 8 == 0;
 }
 
 // Tile of a product, in 16 x 16 tiles of a wave (the block is 2 x 2 waves), and its K slices.  Up to 64 rows:
-// 64 x 64, the most blocks per byte of W.  Else 128 x 256 (less LDS traffic per matrix instruction; two blocks fit a
-// CU) where the grid is at least four rounds of those 512 places, so that a last, partly filled round costs little;
-// else 128 x 128 or 128 x 96 (three blocks a CU).  Measured on the 2B gate/up product: 930 against 790 TFLOP/s at
-// 8192 rows, 700 against 790 at 2048; at 64 rows 35 us with 64 x 64 tiles against 45 us with 128 x 128.
+// 64 x 64, the most blocks per byte of W.  Else 128 x 128 or 128 x 96 (three blocks a CU), by the loop that loads
+// straight into LDS where K allows it; the register-staged loop also has 128 x 256 tiles (less LDS traffic per matrix
+// instruction; two blocks fit a CU) for grids of at least four rounds of those 512 places (2B gate/up, register-staged:
+// 930 against 790 TFLOP/s at 8192 rows, 700 against 790 at 2048).
 struct Tile { int tm, tn; };
 struct Plan { Tile tile; int splits; bool direct = false; };
 
@@ -308,14 +320,27 @@ static int small_tile_splits(const GemmArgs& a, long blocks) {
     return s < 1 ? 1 : s;
 }
 
-// A grid that does not fill the chip's 256 CUs evenly runs as long as its fullest CU: the time of (tile, slices) is
-// taken as the most blocks a CU gets x a block's k steps (a 128 x 96 block costs 0.8 of a 128 x 128 one: fewer products,
-// more LDS traffic for each), plus what writing and reading a further float32 slice of Y costs.  In units of a
-// 128 x 128 block's k step, fitted to the 2B down product at 2,048 rows (288 tiles of 128 x 128: 184 us whole, 140 us
-// in two slices, 115 us as 384 tiles of 128 x 96 in two slices, which is exactly three blocks a CU).
+// The loop that loads straight into LDS takes whole k steps of 64 and 32-bit byte offsets of rows
+static bool direct_ok(const GemmArgs& a) {
+    return a.K % BK == 0 && (long)(a.M > a.N ? a.M : a.N) * a.K * 2 < (1L << 32);
+}
+
+// A grid that does not fill the chip's 256 CUs evenly runs as long as its fullest CU, and a CU holds three blocks at
+// a time.  Microseconds per k step of the blocks a CU gets, with the loads straight into LDS: 1.43 for three blocks
+// together, 1.17 for two, 1.0 for one alone (2B shapes: gate/up at 2,048 rows, nine blocks a CU, 36 steps: 155 us;
+// qkv, two blocks: 42 us; o, 288 tiles: 37 us); a 128 x 96 block costs 0.8 of a 128 x 128 one.
+static double direct_step_us(long blocks) {
+    const long per_cu = tp_cdiv(blocks, 256), rest = per_cu % 3;
+    return (double)(per_cu / 3) * 1.43 + (rest == 2 ? 1.17 : rest == 1 ? 1.0 : 0.0);
+}
+
+// (tile, K slices) of a product of many rows: the cheapest by the model above (register-staged loop, for a K that is
+// no multiple of 64: the most blocks a CU gets x 0.64 us a step, fitted to the 2B down product at 2,048 rows), plus
+// what writing and reading a further float32 slice of Y costs.
 static Plan mid_tile_plan(const GemmArgs& a, bool may_slice) {
     const double step_us = 0.64, slice_us = (double)a.M * a.N * 8 / 4.0e6;
-    Plan best{{4, 4}, 1};
+    const bool direct = direct_ok(a) && a.algo != 7;
+    Plan best{{4, 4}, 1, direct};
     double best_cost = 1e30;
     for (int tn = 4; tn >= 3; tn--) {
         if (tn == 3 && a.epilogue == TP_EPI_GATED) continue;             // gate and up columns come in pairs of tiles
@@ -323,36 +348,30 @@ static Plan mid_tile_plan(const GemmArgs& a, bool may_slice) {
         for (int s = 1; s <= (may_slice ? 4 : 1); s++) {
             if (s > 1 && a.K / s < 512) break;
             const double k_steps = (double)tp_cdiv(tp_cdiv(a.K, s), BK);
-            const double cost = (double)tp_cdiv(tiles * s, 256) * k_steps * step_us * (tn == 3 ? 0.8 : 1.0) + (s - 1) * slice_us;
-            if (cost < best_cost * 0.97) { best_cost = cost; best = {{4, tn}, s, false}; }      // a tie stays with the earlier, plainer plan
-        }
-    }
-    // the loop with loads straight into LDS: 128 x 128 tiles, two blocks a CU (64 KB of LDS each), so rounds of 512
-    // blocks; a k step takes 1.15 us whether a CU holds one block or two (at 2,048 rows: o 288 blocks 35 us, qkv 512
-    // blocks 43 us, down 288 blocks 134 us; at 4,096 rows: qkv 1,024 blocks 83 us, o 576 blocks 66 us)
-    if (a.K % BK == 0 && a.algo != 7 && (long)(a.M > a.N ? a.M : a.N) * a.K * 2 < (1L << 32)) {    // (32-bit row offsets)
-        const long tiles = (long)tp_cdiv(a.M, 128) * tp_cdiv(a.N, 128);
-        for (int s = 1; s <= (may_slice ? 4 : 1); s++) {
-            if (s > 1 && a.K / s < 512) break;
-            const double k_steps = (double)tp_cdiv(tp_cdiv(a.K, s), BK);
-            const double cost = (double)tp_cdiv(tiles * s, 512) * k_steps * 1.15 + 2.0 + (s - 1) * slice_us;
-            if (cost < best_cost * 0.97) { best_cost = cost; best = {{4, 4}, s, true}; }
+            // a grid of at most one block a CU is faster by the register-staged loop (0.85 us a step against 1.0:
+            // 128 x 96 tiles at 512 rows, 2B shapes: qkv 30.7 against 35.5 us, down 102 against 119)
+            const bool d = direct && tiles * s > 256;
+            const double per_step = d ? direct_step_us(tiles * s) : tiles * s <= 256 ? 0.85 : (double)tp_cdiv(tiles * s, 256) * step_us;
+            const double cost = per_step * k_steps * (tn == 3 ? 0.8 : 1.0) + (s - 1) * slice_us;
+            if (cost < best_cost * 0.97) { best_cost = cost; best = {{4, tn}, s, d}; }   // a tie stays with the earlier, plainer plan
         }
     }
     return best;
 }
 
 static Plan plan_of(const GemmArgs& a) {
-    const bool may_slice = a.defer && a.epilogue == TP_EPI_NONE && a.algo != 6 && a.algo != 7;
+    const bool may_slice = a.defer && a.epilogue == TP_EPI_NONE && a.algo < 6;
     if (a.algo == 6) return {{4, 8}, 1};
-    if (a.algo == 8) return {{4, 4}, 1, true};
     if (a.algo == 7) return {{4, a.epilogue == TP_EPI_GATED ? 4 : 3}, 1};
+    if (a.algo == 8) return {{4, 4}, 1, true};
+    if (a.algo == 9) return {{4, a.epilogue == TP_EPI_GATED ? 4 : 3}, 1, true};
     // the logits of 64 rows: 250 us with 128 x 128, 275 with 64 x 64; up to 256 rows of a narrow product: 128 x 128
     // tiles would leave most CUs idle (down at 128 rows: 44 us on 72 blocks, against 15 us at 64 rows on 576 blocks
     // of 64 x 64; at 512 rows 128 x 128 wins again)
     if ((a.M <= 64 && !(a.M > 32 && a.N >= 32768)) || (a.M <= 256 && (long)tp_cdiv(a.M, 128) * tp_cdiv(a.N, 128) < 256))
         return {{2, 2}, may_slice ? small_tile_splits(a, (long)tp_cdiv(a.M, 64) * tp_cdiv(a.N, 64)) : 1};
-    if ((long)tp_cdiv(a.M, 128) * tp_cdiv(a.N, 256) >= 2048) return {{4, 8}, 1};
+    // register-staged loop only: 128 x 256 tiles from four rounds of their 512 places on
+    if (!direct_ok(a) && (long)tp_cdiv(a.M, 128) * tp_cdiv(a.N, 256) >= 2048) return {{4, 8}, 1};
     return mid_tile_plan(a, may_slice);
 }
 
@@ -373,14 +392,18 @@ static void mfma_launch(const GemmArgs& a, void* y, int out_dtype, int splits, i
 }
 
 template <int EPI>
-static int mfma_launch_direct(const GemmArgs& a, void* y, int out_dtype, int splits, int kps) {
-    static const hipError_t attr = hipFuncSetAttribute((const void*)gemm_mfma_direct_k<EPI>, hipFuncAttributeMaxDynamicSharedMemorySize, 65536);
-    TP_REQUIRE(attr == hipSuccess, "tiled product: 64 KB of LDS refused (%s)", hipGetErrorString(attr));
-    const int m_tiles = tp_cdiv(a.M, 128), n_tiles = tp_cdiv(a.N, 128);
+static void mfma_launch_direct(const GemmArgs& a, Tile t, void* y, int out_dtype, int splits, int kps) {
+    const int m_tiles = tp_cdiv(a.M, 128), n_tiles = tp_cdiv(a.N, 32 * t.tn);
     dim3 grid((unsigned)(m_tiles * n_tiles), splits);
-    gemm_mfma_direct_k<EPI><<<grid, 256, 65536, a.stream>>>((const bf16_t*)a.x, (const bf16_t*)a.w, y, a.M, a.N, a.K, m_tiles,
-                                                             out_dtype, a.cap, a.units, kps);
-    return 0;
+    const int xcd_panels = (long)m_tiles * n_tiles >= 1024 ? 1 : 0;
+    if (t.tn == 3) {
+        if constexpr (EPI != TP_EPI_GATED)
+            gemm_mfma_direct_k<EPI, 3><<<grid, 256, 0, a.stream>>>((const bf16_t*)a.x, (const bf16_t*)a.w, y, a.M, a.N, a.K, m_tiles,
+                                                                   out_dtype, a.cap, a.units, kps, xcd_panels);
+    } else {
+        gemm_mfma_direct_k<EPI, 4><<<grid, 256, 0, a.stream>>>((const bf16_t*)a.x, (const bf16_t*)a.w, y, a.M, a.N, a.K, m_tiles,
+                                                               out_dtype, a.cap, a.units, kps, xcd_panels);
+    }
 }
 
 template <int EPI>
@@ -405,16 +428,15 @@ int gemm_mfma_launch(const GemmArgs& a) {
         TP_REQUIRE(a.workspace && a.workspace_bytes >= need, "tiled product: workspace of %zu bytes, %zu needed", a.workspace_bytes, need);
         const int kstep = t.tm == 2 ? SMALL_KS : BK;
         const int kps = tp_cdiv(tp_cdiv(a.K, splits), kstep) * kstep;
-        if (plan.direct) { if (int rc = mfma_launch_direct<TP_EPI_NONE>(a, a.workspace, TP_F32, tp_cdiv(a.K, kps), kps)) return rc; }
+        if (plan.direct) mfma_launch_direct<TP_EPI_NONE>(a, t, a.workspace, TP_F32, tp_cdiv(a.K, kps), kps);
         else mfma_launch_tile<TP_EPI_NONE>(a, t, a.workspace, TP_F32, tp_cdiv(a.K, kps), kps);
         return tp_check_launch("linear (tiled kernel, K slices)");
     }
     if (plan.direct) {
-        int rc;
-        if (a.epilogue == TP_EPI_GATED) rc = mfma_launch_direct<TP_EPI_GATED>(a, a.y, a.out_dtype, 1, a.K);
-        else if (a.epilogue == TP_EPI_SOFTCAP) rc = mfma_launch_direct<TP_EPI_SOFTCAP>(a, a.y, a.out_dtype, 1, a.K);
-        else rc = mfma_launch_direct<TP_EPI_NONE>(a, a.y, a.out_dtype, 1, a.K);
-        return rc ? rc : tp_check_launch("linear (tiled kernel, loads into LDS)");
+        if (a.epilogue == TP_EPI_GATED) mfma_launch_direct<TP_EPI_GATED>(a, t, a.y, a.out_dtype, 1, a.K);
+        else if (a.epilogue == TP_EPI_SOFTCAP) mfma_launch_direct<TP_EPI_SOFTCAP>(a, t, a.y, a.out_dtype, 1, a.K);
+        else mfma_launch_direct<TP_EPI_NONE>(a, t, a.y, a.out_dtype, 1, a.K);
+        return tp_check_launch("linear (tiled kernel, loads into LDS)");
     }
     if (a.epilogue == TP_EPI_GATED) mfma_launch_tile<TP_EPI_GATED>(a, t, a.y, a.out_dtype, 1, a.K);
     else if (a.epilogue == TP_EPI_SOFTCAP) mfma_launch_tile<TP_EPI_SOFTCAP>(a, t, a.y, a.out_dtype, 1, a.K);

@@ -87,7 +87,7 @@ class HipOps:
         _bind(self.lib, _CORE_SIGS)
         self._attn = {}
         self._sample_ws = {}
-        self.force_linear = 0           # tests: 1 plain, 2 skinny, 3 tiled (6: its wide tile, 7: its 128 x 96 tile, 8: loads into LDS), 4 multiply-adds (1-2 rows)
+        self.force_linear = 0           # tests: 1 plain, 2 skinny, 3 tiled (6: its wide tile, 7: its 128 x 96 tile, 8, 9: loads into LDS, 128 x 128 and 128 x 96), 4 multiply-adds (1-2 rows)
         self.force_plain_attention = False
 
     # ---- helpers -----------------------------------------------------------------------------------
