@@ -311,10 +311,13 @@ bool gemm_mfma_supports(const GemmArgs& a) {
 struct Tile { int tm, tn; };
 struct Plan { Tile tile; int splits; bool direct = false; };
 
-// K slices of a product of few rows, which is bound by reading W and wants every CU streaming
+// K slices of a product of few rows, which is bound by reading W and wants every CU streaming.  From 17 rows on one
+// block a CU: more slices cost their consumer more than they gain (a 2B decode step of 64 sequences takes 3.52 ms
+// with 640 blocks, 3.34 with 256, 3.54 with 128).  Up to 16 rows the slices are small and the large matrices that
+// come here want more blocks (a 27B step of 8 sequences: 13.6 ms with 640 blocks, 14.5 with 256).
 static int small_tile_splits(const GemmArgs& a, long blocks) {
     if (blocks >= 512 || a.K < 512) return 1;
-    int s = (int)tp_cdiv(640, blocks);
+    int s = (int)tp_cdiv(a.M > 16 ? 256 : 640, blocks);
     if (s > a.K / 256) s = a.K / 256;
     if (s > 16) s = 16;
     return s < 1 ? 1 : s;
