@@ -1,14 +1,17 @@
-// bf16 product for many rows (prefill): LDS-tiled, on the matrix cores, fp32 accumulation.
+// bf16 product for many rows (prefill) and for few rows of a wide or large matrix: LDS-tiled, on the matrix cores,
+// fp32 accumulation.
 //
-// Block: 256 threads = 4 waves in a 2 x 2 arrangement over a 128 x 128 (or 128 x 256) tile of Y; each wave owns
-// 64 x 64 = 4 x 4 (or 4 x 8) tiles of v_mfma_f32_16x16x32_bf16.  W rows are the A operand and X rows the B operand
-// (both are contiguous along k, which is what the instruction wants per lane), so a lane ends up with
-// 4 consecutive columns of one row of Y (one 8- or 16-byte store), and with the gate and the up column of the same
-// unit in two accumulators of the same lane (the packed gate/up matrix alternates 16 gate rows and 16 up rows).
-// K is walked in steps of 64 through one LDS buffer; the next step's global loads are issued before the
-// current step's products and written to LDS after them.  The 16-byte chunks of an LDS row are stored at
-// chunk ^ (row & 7) (rows of 128 bytes; ^ (row & 15) in rows of 256), so that the 16 rows a fragment read touches spread over the banks (measured: bank
-// conflicts fall from a third of the LDS cycles with padded rows to a few per cent).
+// Block: 256 threads = 4 waves in a 2 x 2 arrangement over a tile of Y (128 x 128, 128 x 96, 128 x 256 or 64 x 64); each
+// wave owns TM x TN tiles of v_mfma_f32_16x16x32_bf16.  W rows are the A operand and X rows the B operand (both are
+// contiguous along k, which is what the instruction wants per lane), so a lane ends up with 4 consecutive columns of
+// one row of Y (one 8- or 16-byte store), and with the gate and the up column of the same unit in two accumulators of
+// the same lane (the packed gate/up matrix alternates 16 gate rows and 16 up rows).
+// K is walked in steps through one LDS buffer (three blocks fit a CU).  Two loops: gemm_mfma_direct_k loads a step's
+// tile from global memory straight into LDS while the step before is multiplied out of registers; gemm_mfma_k issues
+// the next step's global loads into registers before the current step's products and writes them to LDS after them
+// (any K, any tile).  The 16-byte chunks of an LDS row are stored at chunk ^ (row & 7) (rows of 128 bytes; ^ (row & 15)
+// in rows of 256), so that the 16 rows a fragment read touches spread over the banks (measured: bank conflicts fall
+// from a third of the LDS cycles with padded rows to a few per cent).
 // Consecutive block ids walk the M tiles of one N tile, so blocks in flight together share W tiles (large grids:
 // per XCD, see the kernel).
 #include "gemm.h"
