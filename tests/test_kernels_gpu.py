@@ -50,7 +50,9 @@ def test_rms_norm(ops, din, dout, m, d):
 @pytest.mark.parametrize("post,nxt", [(True, True), (True, False), (False, True), (False, False)])
 @pytest.mark.parametrize("m,d", [(1, 64), (5, 88), (4, 3584),
                                  # many rows: four elements per lane, one width for each of its forms and their edges
-                                 (130, 88), (200, 1000), (150, 2304), (140, 3072), (129, 4608), (130, 8192), (131, 8200), (130, 90)])
+                                 (130, 88), (200, 1000), (150, 2304), (140, 3072), (129, 4608), (130, 8192), (131, 8200), (130, 90),
+                                 # few rows of many chunks: a chunk a lane, every form and its edges
+                                 (8, 1028), (3, 2304), (64, 2560), (5, 2564), (2, 4096), (7, 4608), (9, 5120), (4, 5124), (6, 8192)])
 def test_add_rms_norm(ops, dt, post, nxt, m, d):
     stream = randn(m, d, seed=3, scale=2.0)
     rows = randn(m, d, dtype=DT[dt], seed=4, scale=5.0)
