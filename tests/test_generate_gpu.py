@@ -127,3 +127,22 @@ def test_graphs_follow_a_sequence_across_their_length_bound(folders):
         b = graphed.step(gs, step_toks).clone()
         assert rel_l2(b, a) < 3e-3, step
     assert len(graphed.by_batch) == 2
+
+
+def test_decode_loop_with_and_without_graph(folders):
+    """The device-resident greedy loop: the graph that also picks the tokens gives the ids of eager steps and argmax."""
+    from .gpu_engine import load_gpu_model
+    from trapetum_amd.engine.decode_loop import DecodeLoop
+    model, cfg = load_gpu_model(folders["B"], "bfloat16")
+    prompts = [random_tokens(n, cfg.vocab_size, 70 + i) for i, n in enumerate((7, 19, 33))]
+    runs = []
+    for use_graph in (False, True):
+        cache = model.new_cache(max_tokens=1024, page_size=16)
+        loop = DecodeLoop(model, cache, use_graph=use_graph)
+        ids = [loop.start(prompts).cpu().tolist()]
+        for _ in range(20):
+            ids.append(loop.step().cpu().tolist())
+            torch.randn(32, 32, device="cuda:0").sum().item()       # unrelated eager work between replays
+        loop.finish()
+        runs.append(ids)
+    assert runs[0] == runs[1]

@@ -11,7 +11,7 @@ class DecodeLoop:
     def __init__(self, model, cache, use_graph=True):
         self.model = model
         self.cache = cache
-        self.graphed = GraphedDecode(model, cache) if use_graph else None
+        self.graphed = GraphedDecode(model, cache, greedy=True) if use_graph else None
         self.slots = []
         self.tokens = None
 
@@ -23,11 +23,12 @@ class DecodeLoop:
         return self.tokens
 
     def step(self):
-        if self.graphed is not None:
-            logits = self.graphed.step(self.slots, self.tokens)
+        if self.graphed is not None:               # the graph picks the tokens and leaves them where its next replay reads them
+            self.graphed.step(self.slots, self.tokens)
+            self.tokens = self.graphed.chosen
         else:
             logits = self.model.step(self.cache, self.slots, self.tokens)
-        self.tokens = self.model.rt.ops.argmax(logits)
+            self.tokens = self.model.rt.ops.argmax(logits)
         return self.tokens
 
     def finish(self):

@@ -19,11 +19,16 @@ class _Captured:
 
 
 class GraphedDecode:
-    def __init__(self, model, cache):
+    def __init__(self, model, cache, greedy=False):
+        """greedy: the graph also picks every sequence's next token (argmax) and leaves it where the next replay
+        reads its tokens, so that a greedy loop needs neither a launch nor a copy between replays; `chosen` is that
+        tensor after a step."""
         if model.rt.device.type != "cuda":
             raise RuntimeError("HIP graphs need the GPU")
         self.model = model
         self.cache = cache
+        self.greedy = greedy
+        self.chosen = None
         self.by_batch = {}
 
     def step(self, slots, tokens):
@@ -48,15 +53,21 @@ class GraphedDecode:
             tokens_static.copy_(tok)
             ctx = StepContext(model.rt, cache, slots, counts, starts, want, static=static)
             logits = model.run(ctx, tokens_static)          # this step, eagerly; also loads what capture must not
+            if self.greedy:
+                model.rt.ops.argmax(logits, out=tokens_static)
             torch.cuda.synchronize(model.rt.device)
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
                 captured_logits = model.run(ctx, tokens_static)
+                if self.greedy:
+                    model.rt.ops.argmax(captured_logits, out=tokens_static)
             self.by_batch[b] = _Captured(static, tokens_static, ctx, graph, captured_logits)
+            self.chosen = tokens_static
             return logits
         flat, _ = step_arrays(cache, slots, counts, starts, want, cap.static.table_widths)
         cap.static.fill(flat)
         if tok.data_ptr() != cap.tokens.data_ptr():
             cap.tokens.copy_(tok)
         cap.graph.replay()
+        self.chosen = cap.tokens
         return cap.logits

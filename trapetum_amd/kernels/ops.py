@@ -387,11 +387,17 @@ class HipOps:
         return out
 
     # ---- token choice -------------------------------------------------------------------------------------
-    def argmax(self, logits):
+    def argmax(self, logits, out=None):
+        """Smallest index of the largest value per row, int32; into `out` if given."""
         self._dev(logits)
         if logits.dtype != torch.float32 or logits.dim() != 2 or not logits.is_contiguous():
             raise KernelError("argmax: logits must be contiguous float32 [rows, vocab]")
-        out = torch.empty(logits.shape[0], dtype=torch.int32, device=self.device)
+        if out is None:
+            out = torch.empty(logits.shape[0], dtype=torch.int32, device=self.device)
+        else:
+            self._dev(out)
+            if out.dtype != torch.int32 or out.shape != (logits.shape[0],) or not out.is_contiguous():
+                raise KernelError("argmax: the output must be contiguous int32 [rows]")
         nbytes = self.lib.tp_argmax_workspace_bytes(logits.shape[0], logits.shape[1])
         ws = torch.empty(nbytes, dtype=torch.uint8, device=self.device) if nbytes else None
         self._call(self.lib, "tp_argmax", logits.data_ptr(), logits.shape[0], logits.shape[1], out.data_ptr(),
