@@ -46,14 +46,25 @@ def build_dir():
         return d
 
 
-def _headers():
-    return sorted(f for f in os.listdir(CSRC) if f.endswith(".h"))
+def _headers(sources):
+    """The headers of csrc/ that the sources include, directly or through one another."""
+    seen, todo = set(), list(sources)
+    while todo:
+        with open(os.path.join(CSRC, todo.pop()), "r", errors="replace") as f:
+            for line in f:
+                line = line.strip()
+                if line.startswith("#include \""):
+                    name = line.split('"')[1]
+                    if name not in seen and os.path.isfile(os.path.join(CSRC, name)):
+                        seen.add(name)
+                        todo.append(name)
+    return sorted(seen)
 
 
 def _stamp(sources, defines):
     h = hashlib.sha256()
     h.update(" ".join(FLAGS + defines).encode())
-    for name in list(sources) + _headers():
+    for name in list(sources) + _headers(sources):
         with open(os.path.join(CSRC, name), "rb") as f:
             h.update(name.encode())
             h.update(f.read())
