@@ -1,5 +1,7 @@
 // Token choice on the device: argmax, repetition penalty, temperature / top-k / top-p sampling.
 #include "common.h"
+#include "no_alloc.h"
+#include <mutex>
 
 // ---- argmax: the smallest index among the largest values (strict '>' scan in the reference:
 // runtime/src/lib.rs:1376-1380; device twin runtime/cuda/codebook_gemv.cu:548-591).  One block per row. ----
@@ -99,6 +101,57 @@ extern "C" int tp_argmax(const float* logits, int B, int V, int* out, void* work
     if (int rc = tp_check_launch("argmax (parts)")) return rc;
     argmax_final_k<<<B, 64, 0, s>>>(pval, pidx, parts, out);
     return tp_check_launch("argmax (final)");
+}
+
+// ---- argmax for callers that cannot allocate (declared in no_alloc.h) -------------------------------------------
+// The two-stage form above with the parts' winners in a file-scope device array instead of a caller's workspace.
+// Every GPU the library runs on holds its own copy of the array (128 KiB) until the process ends; in host code the
+// array's name is only a handle, so its device address is asked for once per device (hipGetSymbolAddress with that
+// device current) and kept.  Nothing in the array has to start at zero: stage 2 reads exactly the B * parts pairs
+// that stage 1 of the same call wrote.  All calls on one GPU share the array: calls that overlap there (two
+// streams, two threads) race.
+static __device__ __align__(256) unsigned char scratch[TP_ARGMAX_NO_ALLOC_SCRATCH_BYTES];
+
+namespace {
+constexpr int NO_ALLOC_MAX_DEVICES = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[NO_ALLOC_MAX_DEVICES];        // per device: where that GPU's copy of `scratch` lies
+
+int scratch_address(void** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return tp_fail("argmax_no_alloc: no current device: %s", hipGetErrorString(e));
+    TP_REQUIRE(dev >= 0 && dev < NO_ALLOC_MAX_DEVICES, "argmax_no_alloc: device %d is beyond the %d this library keeps track of", dev, NO_ALLOC_MAX_DEVICES);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr)
+            return tp_fail("argmax_no_alloc: the scratch array's address on device %d is not available: %s", dev, hipGetErrorString(e));
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = g_scratch_ptr[dev];
+    return 0;
+}
+}  // namespace
+
+extern "C" int tp_argmax_no_alloc(const float* logits, int B, int V, int* out, void* stream) {
+    TP_REQUIRE(logits && out, "argmax_no_alloc: logits and output must be given");
+    TP_REQUIRE(B > 0 && V > 0, "argmax_no_alloc: empty shape B=%d V=%d", B, V);
+    TP_REQUIRE(B <= TP_ARGMAX_NO_ALLOC_MAX_ROWS, "argmax_no_alloc: %d rows exceed the %d that the fixed scratch array holds",
+               B, TP_ARGMAX_NO_ALLOC_MAX_ROWS);
+    static_assert((size_t)TP_ARGMAX_NO_ALLOC_MAX_ROWS * TP_ARGMAX_NO_ALLOC_PARTS * 8 <= TP_ARGMAX_NO_ALLOC_SCRATCH_BYTES,
+                  "the scratch array must hold a (value, index) pair per row and part");
+    void* base = nullptr;
+    if (int rc = scratch_address(&base)) return rc;
+    const int parts = TP_ARGMAX_NO_ALLOC_PARTS;
+    float* pval = (float*)base;
+    int* pidx = (int*)(pval + (size_t)B * parts);
+    hipStream_t s = (hipStream_t)stream;
+    argmax_part_k<<<dim3(parts, B), 256, 0, s>>>(logits, V, tp_cdiv(V, parts), pval, pidx);
+    if (int rc = tp_check_launch("argmax_no_alloc (parts)")) return rc;
+    argmax_final_k<<<B, 64, 0, s>>>(pval, pidx, parts, out);
+    return tp_check_launch("argmax_no_alloc (final)");
 }
 
 // ---- repetition penalty: every distinct recent token once, z / penalty if z > 0 else z * penalty
