@@ -5,6 +5,7 @@ import torch
 from .cpu_engine import load_cpu_model
 from .plain import gemma2_plain as plain
 from .tiny import CONFIGS, make_folder, random_tokens, rel_l2
+from . import trace_schedules as ts
 
 
 @pytest.fixture(scope="module", params=["A", "B", "C"])
@@ -65,3 +66,20 @@ def test_unequal_batches_and_slot_reuse(setup):
             ref = plain.forward(pcfg, pw, seqs[i][:n])[lens[i] - 1:n]
             assert rel_l2(torch.stack(got[i]), ref) < 2e-5, (batch, i)
     assert cache.live_slots() == []
+
+
+@pytest.mark.parametrize("page_size", [16, 64])
+def test_portions_and_joining_requests(setup, page_size):
+    """A sequence fed in portions of any size, and requests that join a running batch, give the logits of whole
+    sequences.  With pages of 16 the windows' rings have no row to spare (B: window 16 in a ring of 16), so a
+    portion overwrites ring rows that its own earlier queries still see."""
+    model, cfg, pcfg, pw = setup
+    requests = {f"r{i}": random_tokens(n, cfg.vocab_size, 40 + i) for i, n in enumerate([70, 9, 41, 2, 35])}
+    ref = {rid: plain.forward(pcfg, pw, t) for rid, t in requests.items()}
+    for steps in (ts.chunked(requests, [16]), ts.chunked(requests, [1, 7, 32]), ts.chunked(requests, [2, 17, 3]),
+                  ts.joining(requests), ts.joining(requests, every=1, burst=9)):
+        cache = model.new_cache(max_tokens=ts.held_tokens(steps, page_size), page_size=page_size)
+        got = ts.collect(steps, ts.run_on_model(model, cache, steps), cfg.vocab_size)
+        assert cache.live_slots() == []
+        for rid in requests:
+            assert rel_l2(torch.from_numpy(got[rid]), ref[rid]) < 2e-5, rid

@@ -4,6 +4,7 @@ import torch
 
 from .plain import gemma2_plain as plain
 from .tiny import make_folder, random_tokens, rel_l2
+from . import trace_schedules as ts
 
 pytestmark = pytest.mark.gpu
 TOL = {"float32": 1e-5, "bfloat16": 2e-2}
@@ -101,3 +102,20 @@ def test_steps_repeat_bit_for_bit(setup):
             rows.append(model.step(cache, slots, [s[n + step] for s, n in zip(seqs, lens)]))
         runs.append(torch.cat(rows).cpu())
     assert torch.equal(runs[0], runs[1])
+
+
+@pytest.mark.parametrize("page_size", [16, 64])
+def test_portions_and_joining_requests(setup, page_size):
+    """A sequence fed in portions of any size, and requests that join a running batch, give the logits of whole
+    sequences.  With pages of 16 the windows' rings have no row to spare (B: window 16 in a ring of 16), so a
+    portion overwrites ring rows that its own earlier queries still see."""
+    model, cfg, pcfg, pw, tol = setup
+    requests = {f"r{i}": random_tokens(n, cfg.vocab_size, 40 + i) for i, n in enumerate([70, 9, 41, 2, 35])}
+    ref = {rid: plain.forward(pcfg, pw, t) for rid, t in requests.items()}
+    for steps in (ts.chunked(requests, [16]), ts.chunked(requests, [1, 7, 32]), ts.chunked(requests, [2, 17, 3]),
+                  ts.joining(requests), ts.joining(requests, every=1, burst=9)):
+        cache = model.new_cache(max_tokens=ts.held_tokens(steps, page_size), page_size=page_size)
+        got = ts.collect(steps, ts.run_on_model(model, cache, steps), cfg.vocab_size)
+        assert cache.live_slots() == []
+        for rid in requests:
+            assert rel_l2(torch.from_numpy(got[rid]), ref[rid]) < tol, rid

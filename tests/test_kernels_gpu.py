@@ -289,6 +289,73 @@ def test_attention_prefill_many_tiles(ops, H, KV, hd, lens, window, cap):
     assert rel_l2(got.reshape(m, H, hd), ref) < 8e-3
 
 
+EXTEND_CASES = [
+    # H, KV, hd, lens, starts (what the cache already holds), page, window, rows_cap, cap
+    (4, 2, 16, (25, 11, 17), (20, 0, 16), 16, 8, 16, 50.0),
+    (6, 1, 32, (50, 9, 23, 40), (17, 8, 0, 1), 16, 16, 16, 20.0),         # a ring without a row to spare
+    (3, 3, 48, (70, 3), (64, 2), 16, 5, 16, 8.0),
+    (8, 4, 256, (330, 64), (130, 63), 64, 0, 0, 50.0),
+    (8, 4, 256, (700,), (451,), 64, 128, 128, 0.0),                       # the portion is longer than the ring
+    (2, 2, 80, (33, 50), (0, 31), 16, 0, 0, 0.0),
+    (16, 2, 128, (1300, 17, 129), (1234, 0, 128), 64, 512, 512, 30.0),
+    (32, 1, 64, (90,), (89,), 16, 0, 0, 0.0),
+]
+
+
+@pytest.mark.parametrize("plain", [True, False])
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("H,KV,hd,lens,starts,page,window,rows_cap,cap", EXTEND_CASES)
+def test_attention_over_cached_positions_and_the_steps_rows(ops, plain, dt, H, KV, hd, lens, starts, page, window, rows_cap, cap):
+    """A step that continues sequences by several tokens: the cached positions are copied out of the (ring) cache,
+    the step's rows are rotated, cached and added to them, and the queries attend over both.  Against whole-sequence
+    attention of the reference; afterwards the cache holds what a whole-sequence step would have left."""
+    from trapetum_amd.engine.batch import KeyGeometry
+    if dt == "f32" and not plain:
+        pytest.skip("float32 runs on the plain kernel only")
+    n_pages = 64
+    c = build_cache_case(DT[dt], H, KV, hd, lens, page, rows_cap, n_pages, 50)
+    scale = 1.0 / math.sqrt(hd * 0.9)
+    q_ref, k_ref = c["q"].cpu().clone(), c["k"].cpu().clone()
+    pools_ref = [torch.zeros(n_pages, KV, page, hd, dtype=DT[dt]) for _ in range(2)]
+    ref_ops.rope_kv_write(q_ref, k_ref, c["v"].cpu(), H, KV, hd, c["inv_freq"], hd, c["row_seq"], c["row_pos"],
+                          c["new_len"], c["table"], pools_ref[0], pools_ref[1], rows_cap)
+    ref = ref_ops.attention_prefill(q_ref, k_ref, c["v"].cpu(), H, KV, hd, c["cu"], max(lens), scale, cap, window, torch.float32)
+    # what earlier steps left: positions below `starts`, written as one step per sequence set
+    pools = [torch.full((n_pages, KV, page, hd), 7.0, dtype=DT[dt], device=DEV) for _ in range(2)]
+    first = torch.cat([torch.arange(int(c["cu"][i]), int(c["cu"][i]) + s) for i, s in enumerate(starts)]).long()
+    if first.numel():
+        ops.rope_kv_write(c["q"][first.to(DEV)].contiguous(), c["k"][first.to(DEV)].contiguous(), c["v"][first.to(DEV)].contiguous(),
+                          H, KV, hd, c["inv_freq"].to(DEV), hd, c["row_seq"][first].to(DEV), c["row_pos"][first].to(DEV),
+                          torch.tensor(starts, dtype=torch.int32, device=DEV), c["table"].to(DEV), pools[0], pools[1], rows_cap)
+    # the step: positions starts[i] .. lens[i] - 1 of every sequence
+    counts = [n - s for n, s in zip(lens, starts)]
+    rows = torch.cat([torch.arange(int(c["cu"][i]) + s, int(c["cu"][i + 1])) for i, s in enumerate(starts)]).long()
+    q, k, v = (c[name][rows.to(DEV)].contiguous() for name in ("q", "k", "v"))
+    cu = torch.tensor([0] + list(torch.tensor(counts).cumsum(0)), dtype=torch.int32, device=DEV)
+    keys = KeyGeometry(starts, counts, window)
+    keys.cu_keys_dev, keys.key_row0_dev, keys.prefix_lo_dev = (torch.tensor(a, dtype=torch.int32, device=DEV)
+                                                                for a in (keys.cu_keys, keys.key_row0, keys.prefix_lo))
+    ops.force_plain_attention = plain
+    try:
+        gk, gv = ops.gather_kv_prefix(c["table"].to(DEV), pools[0], pools[1], rows_cap, cu, keys)
+        ops.rope_kv_write(q, k, v, H, KV, hd, c["inv_freq"].to(DEV), hd, c["row_seq"][rows].to(DEV), c["row_pos"][rows].to(DEV),
+                          c["new_len"].to(DEV), c["table"].to(DEV), pools[0], pools[1], rows_cap,
+                          gathered=(gk, gv, keys.key_row0_dev))
+        got = ops.attention_prefill(q, gk, gv, H, KV, hd, cu, max(counts), scale, cap, window, DT[dt],
+                                    row_seq=c["row_seq"][rows].to(DEV), row_pos=c["row_pos"][rows].to(DEV), keys=keys)
+    finally:
+        ops.force_plain_attention = False
+    assert rel_l2(got, ref[rows]) < (3e-6 if dt == "f32" else 8e-3)
+    worst = max(rel_l2(got[i], ref[rows][i]) for i in range(0, len(rows), max(1, len(rows) // 50)))
+    assert worst < (1e-5 if dt == "f32" else 3e-2)
+    # the cache afterwards: every row a whole-sequence step writes holds the same values
+    written = (pools_ref[0] != 0).any(dim=-1)
+    t = 3e-6 if dt == "f32" else 6e-3
+    assert rel_l2(pools[0].cpu()[written], pools_ref[0][written]) < t
+    assert torch.equal(pools[1].cpu()[written], pools_ref[1][written])
+    assert bool((pools[0].cpu()[~written] == 7.0).all())
+
+
 @pytest.mark.parametrize("plain", [True, False])
 @pytest.mark.parametrize("dt", ["f32", "bf16"])
 @pytest.mark.parametrize("H,KV,hd,lens,page,window,rows_cap,cap", ATTN_CASES)

@@ -12,6 +12,7 @@ from trapetum_amd.weights import WeightFolder, load_folder, write_model_folder
 from . import toy_parts
 from .cpu_engine import ref_ops_namespace
 from .tiny import random_tokens, rel_l2
+from . import trace_schedules as ts
 
 
 @pytest.fixture(scope="module")
@@ -67,3 +68,17 @@ def test_toy_whole_stepwise_and_batched(toy):
         step += 1
     for i in range(3):
         assert rel_l2(torch.stack(got[i]), ref[i][lens[i] - 1:]) < 2e-5, i
+
+
+def test_toy_portions_and_joining(toy):
+    """Steps of any shape reach the toy's parts too: the state mixer scans a portion from the state it kept, and the
+    run that reads another run's cache sees the cached positions gathered for that run."""
+    model, weights = toy
+    vocab = toy_parts.TOY["vocab"]
+    requests = {f"r{i}": random_tokens(n, vocab, 60 + i) for i, n in enumerate([33, 5, 18])}
+    ref = {rid: toy_parts.toy_reference(toy_parts.TOY, weights, t) for rid, t in requests.items()}
+    for steps in (ts.chunked(requests, [4, 1, 9]), ts.joining(requests, every=1, burst=5)):
+        cache = model.new_cache(max_tokens=ts.held_tokens(steps, 16), page_size=16)
+        got = ts.collect(steps, ts.run_on_model(model, cache, steps), vocab)
+        for rid in requests:
+            assert rel_l2(torch.from_numpy(got[rid]), ref[rid]) < 2e-5, rid

@@ -11,6 +11,7 @@ from trapetum_amd.weights import WeightFolder, load_folder, write_model_folder
 
 from . import toy_parts
 from .tiny import random_tokens, rel_l2
+from . import trace_schedules as ts
 
 pytestmark = pytest.mark.gpu
 
@@ -53,3 +54,11 @@ def test_toy_model_steps(tmp_path, dtype, tol):
         step += 1
     for i in range(3):
         assert rel_l2(torch.stack(got[i]), ref[i][lens[i] - 1:]) < tol, i
+
+    # steps of any shape: portions, and requests that join a running batch
+    requests = {f"r{i}": q for i, q in enumerate(seqs)}
+    for steps in (ts.chunked(requests, [4, 1, 9]), ts.joining(requests, every=1, burst=5)):
+        cache = model.new_cache(max_tokens=ts.held_tokens(steps, 16), page_size=16)
+        out = ts.collect(steps, ts.run_on_model(model, cache, steps), toy_parts.TOY["vocab"])
+        for i in range(3):
+            assert rel_l2(torch.from_numpy(out[f"r{i}"]), ref[i]) < tol, i

@@ -34,7 +34,9 @@ def test_schedules_agree(folder):
     vocab = pcfg["vocab_size"]
     requests = {f"r{i}": random_tokens(n, vocab, 20 + i) for i, n in enumerate([70, 9, 41, 1, 66])}
     ref = {rid: plain.forward(pcfg, pw, t) for rid, t in requests.items()}
-    for steps in (ts.whole(requests), ts.last_one_by_one(requests, 32), ts.batches(requests, 2)):
+    for steps in (ts.whole(requests), ts.last_one_by_one(requests, 32), ts.batches(requests, 2),
+                  ts.chunked(requests, [16]), ts.chunked(requests, [1, 7, 32]), ts.chunked(requests, [2, 63, 3]),
+                  ts.joining(requests)):
         got = ts.collect(steps, run(folder, steps, ts.held_tokens(steps)), vocab)
         for rid in requests:
             assert rel_l2(torch.from_numpy(got[rid]), ref[rid]) < 2e-5
@@ -49,15 +51,24 @@ def test_cache_is_sized_by_max_tokens(folder):
     run(folder, steps, 192)
 
 
-def test_refused_steps(folder):
+def test_steps_of_any_shape_and_what_is_still_refused(folder):
     r = TraceRunner(folder, "float32", 256, device="cpu", ops=ref_ops_namespace())
     r.run_step({"step": 0, "entries": [{"id": "a", "tokens": [1, 2, 3], "want": []}], "end": []})
-    with pytest.raises(StepError):       # one request continues by two tokens
-        r.run_step({"step": 1, "entries": [{"id": "a", "tokens": [4, 5], "want": []}], "end": []})
-    with pytest.raises(StepError):       # a request joins a batch that has started
-        r.run_step({"step": 1, "entries": [{"id": "a", "tokens": [4], "want": []}, {"id": "b", "tokens": [1, 2], "want": []}], "end": []})
-    assert r.cache.live_slots() == [r.slot_of["a"]] and r.cache.length(r.slot_of["a"]) == 3
+    # a request continues by two tokens; another joins the batch that has started
+    r.run_step({"step": 1, "entries": [{"id": "a", "tokens": [4, 5], "want": []}], "end": []})
+    r.run_step({"step": 2, "entries": [{"id": "a", "tokens": [6], "want": []}, {"id": "b", "tokens": [1, 2], "want": []}], "end": []})
+    assert r.cache.length(r.slot_of["a"]) == 6 and r.cache.length(r.slot_of["b"]) == 2
+    with pytest.raises(TraceError):      # an entry without tokens
+        r.run_step({"step": 3, "entries": [{"id": "a", "tokens": [], "want": []}], "end": []})
+    with pytest.raises(TraceError):      # a wanted place outside the entry's tokens
+        r.run_step({"step": 3, "entries": [{"id": "a", "tokens": [7], "want": [1]}], "end": []})
+    with pytest.raises(StepError):       # a token outside the vocabulary; the newcomer's slot is given back
+        r.run_step({"step": 3, "entries": [{"id": "a", "tokens": [7], "want": []}, {"id": "c", "tokens": [100000], "want": []}], "end": []})
+    assert "c" not in r.slot_of and r.cache.length(r.slot_of["a"]) == 6
+    with pytest.raises(CacheError):      # more tokens than the cache was sized for
+        r.run_step({"step": 3, "entries": [{"id": "a", "tokens": list(range(200)), "want": []}], "end": []})
+    assert r.cache.length(r.slot_of["a"]) == 6
     with pytest.raises(TraceError):
-        r.run_step({"step": 2, "entries": [], "end": ["zz"]})
-    assert r.run_step({"step": 3, "entries": [{"id": "a", "tokens": [4], "want": []}], "end": ["a"]}) is None
+        r.run_step({"step": 4, "entries": [], "end": ["zz"]})
+    assert r.run_step({"step": 5, "entries": [{"id": "a", "tokens": [4], "want": []}], "end": ["a", "b"]}) is None
     assert r.cache.live_slots() == []

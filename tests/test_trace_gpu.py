@@ -43,9 +43,11 @@ def test_replay_schedules_agree_with_plain(which, dtype, tmp_path):
     lens = [70, 41, 97, 5, 33, 1, 64]
     requests = {f"r{i}": random_tokens(n, vocab, 10 + i) for i, n in enumerate(lens)}
     ref = {rid: plain.forward(pcfg, pw, toks) for rid, toks in requests.items()}
-    schedules = {"whole": ts.whole(requests), "tail": ts.last_one_by_one(requests, 32), "batches": ts.batches(requests, 3)}
+    schedules = {"whole": ts.whole(requests), "tail": ts.last_one_by_one(requests, 32), "batches": ts.batches(requests, 3),
+                 "portions of 16": ts.chunked(requests, [16]), "portions of 1, 7, 32": ts.chunked(requests, [1, 7, 32]),
+                 "joining a running batch": ts.joining(requests)}
     for name, steps in schedules.items():
-        out_dir = str(tmp_path / f"out_{name}")
+        out_dir = str(tmp_path / ("out_" + name.replace(" ", "_").replace(",", "")))
         got = ts.collect(steps, replay(folder, dtype, steps, out_dir, ts.held_tokens(steps)), vocab)
         for rid in requests:
             assert got[rid].shape == tuple(ref[rid].shape), (name, rid)

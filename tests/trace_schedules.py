@@ -52,6 +52,47 @@ def batches(requests, batch_size, prefill_fraction=0.5):
     return steps
 
 
+def chunked(requests, sizes):
+    """Each request alone, fed in portions whose sizes cycle through `sizes`; every position wanted."""
+    steps = []
+    for rid, toks in requests.items():
+        at, turn = 0, 0
+        while at < len(toks):
+            n = min(sizes[turn % len(sizes)], len(toks) - at)
+            steps.append({"step": len(steps), "entries": [{"id": rid, "tokens": toks[at:at + n], "want": list(range(n))}],
+                          "end": [rid] if at + n == len(toks) else []})
+            at += n
+            turn += 1
+    return steps
+
+
+def joining(requests, every=2, burst=4):
+    """Requests join a batch that is running: every `every` steps the next request starts with half of its tokens in
+    one portion, while those already running go on by one token, or by `burst` tokens now and then; a request
+    leaves when its tokens run out."""
+    steps = []
+    waiting = list(requests)
+    done, live = {}, []
+    while waiting or live:
+        k = len(steps)
+        entries = []
+        for i, rid in enumerate(live):
+            n = burst if (k + i) % 4 == 0 else 1
+            n = min(n, len(requests[rid]) - done[rid])
+            entries.append({"id": rid, "tokens": requests[rid][done[rid]:done[rid] + n], "want": list(range(n))})
+            done[rid] += n
+        if waiting and (k % every == 0 or not live):
+            rid = waiting.pop(0)
+            n = max(1, (len(requests[rid]) + 1) // 2)
+            entries.append({"id": rid, "tokens": requests[rid][:n], "want": list(range(n))})
+            done[rid] = n
+            live.append(rid)
+        ends = [rid for rid in live if done[rid] == len(requests[rid])]
+        steps.append({"step": k, "entries": entries, "end": ends})
+        live = [rid for rid in live if rid not in ends]
+    return steps
+
+
 def collect(steps, outputs, vocab):
     """outputs: {step: array [wanted, vocab]} -> {request id: array [len, vocab]} in position order."""
     import numpy as np
@@ -79,3 +120,25 @@ def held_tokens(steps, page=64):
         for rid in rec["end"]:
             del held[rid]
     return most
+
+
+def run_on_model(model, cache, steps):
+    """The schedule's steps through model.step on `cache` (any page size); {step: logits [wanted, vocab]} as arrays."""
+    slot_of, out = {}, {}
+    for rec in steps:
+        slots, counts, flat, want, offset = [], [], [], [], 0
+        for e in rec["entries"]:
+            if e["id"] not in slot_of:
+                slot_of[e["id"]] = cache.acquire()
+            slots.append(slot_of[e["id"]])
+            counts.append(len(e["tokens"]))
+            flat.extend(e["tokens"])
+            want.extend(offset + w for w in e.get("want", []))
+            offset += len(e["tokens"])
+        logits = model.step(cache, slots, flat, counts=counts, want=want)
+        if logits is not None:
+            out[rec["step"]] = logits.float().cpu().numpy()
+        for rid in rec["end"]:
+            cache.release(slot_of.pop(rid))
+    assert not slot_of
+    return out

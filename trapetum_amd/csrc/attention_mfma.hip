@@ -1,5 +1,6 @@
 // bf16 attention on the matrix cores for one head size (compiled with -DTP_HD=<head_dim>, a multiple of 16 up
-// to 256): a prefill kernel over the step's own keys and values and a decode kernel over the paged cache.
+// to 256): a prefill kernel over a buffer of keys and values (the step's own rows, behind the cached positions
+// its queries still see when sequences continue) and a decode kernel over the paged cache.
 //
 // Formula as the reference's attn_k (runtime/cuda/codebook_gemv.cu:240-270): score = (q . k) * scale, then
 // cap * tanh(score / cap) if a cap is set, softmax over the visible keys in fp32, weighted sum of v, query head
@@ -51,14 +52,17 @@ __device__ __forceinline__ bf16_t bf16_bits(float f) {
 }  // namespace
 
 // =====================================================================================================
-// prefill: every sequence of the step starts at position 0; keys and values are the step's own rows.
+// prefill: a sequence's keys and values are rows cu_keys[s] .. cu_keys[s + 1] - 1 of k and v, its queries the
+// rows cu_rows[s] .. of q, and the queries are the sequence's LAST positions: with Tk keys and Tq queries the
+// first query stands at key Tk - Tq (0 when every sequence starts in this step and the keys are its own rows;
+// more when cached positions were gathered in front of them).  Only differences of positions count.
 // Block = 64 or 32 queries of one (sequence, head); a wave owns 16 queries.  Key tiles of 32 go through LDS: K as
 // stored (row = key), V transposed (row = head element) with the keys of a tile permuted so that a lane's 8
 // probabilities meet the 8 values of the same keys in one 16-byte LDS read.
 // =====================================================================================================
 struct PrefillArgs {
     const bf16_t* q; long q_stride; const bf16_t* k; long k_stride; const bf16_t* v; long v_stride;
-    int H, KV; const int* cu_rows; float scale, cap; int window; bf16_t* out;
+    int H, KV; const int* cu_rows; const int* cu_keys; float scale, cap; int window; bf16_t* out;
     const bf16_t* vt; long vt_rows;      // V transposed: [kv head][head element][padded key slot], vt_rows slots per row
 };
 
@@ -145,17 +149,19 @@ attn_prefill_k(PrefillArgs a) {
     const bf16_t* Vt = Vt_all + grp * VT_ELEMS;
     // late query tiles see the most keys: they are given the low block ids, which start first
     const int seq = blockIdx.z, h = blockIdx.x % a.H, q0 = (gridDim.x / a.H - 1 - blockIdx.x / a.H) * PQ;
-    const int row0 = a.cu_rows[seq], T = a.cu_rows[seq + 1] - row0;
-    if (q0 >= T) return;
+    // rows of the queries (row0, Tq of them) and of the keys (krow0, T of them); query i stands at key qofs + i
+    const int row0 = a.cu_rows[seq], Tq = a.cu_rows[seq + 1] - row0;
+    if (q0 >= Tq) return;
+    const int krow0 = a.cu_keys[seq], T = a.cu_keys[seq + 1] - krow0, qofs = T - Tq;
     const int kvh = h / (a.H / a.KV);
-    const int qw0 = q0 + wave * 16, qpos = qw0 + c;
+    const int qw0 = qofs + q0 + wave * 16, qpos = qw0 + c;       // in key coordinates
     const bool q_ok = qpos < T;
 
     bf16x8 qf[KSTEPS];
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ks++) {
         const int d0 = ks * 32 + g * 8;
-        qf[ks] = ld_frag(a.q + (size_t)(row0 + (q_ok ? qpos : 0)) * a.q_stride + (size_t)h * HD + d0, q_ok && d0 < HD);
+        qf[ks] = ld_frag(a.q + (size_t)(row0 + (q_ok ? qpos - qofs : 0)) * a.q_stride + (size_t)h * HD + d0, q_ok && d0 < HD);
     }
     if (HDP > HD)                                   // the padding columns of K stay zero for the whole kernel
         for (int i = tid; i < PKEYS * (HDP - HD); i += PTH) {
@@ -173,9 +179,9 @@ attn_prefill_k(PrefillArgs a) {
     const int seen_lo = a.window > 0 ? max(0, qpos - a.window + 1) : 0;
     const unsigned seen_span = (unsigned)max(0, min(qpos, T - 1) - seen_lo);
 
-    int k_lo = a.window > 0 ? max(0, q0 - a.window + 1) : 0;
+    int k_lo = a.window > 0 ? max(0, qofs + q0 - a.window + 1) : 0;
     k_lo &= ~(BKV - 1);
-    const int k_hi = min(T, q0 + PQ);
+    const int k_hi = min(T, qofs + q0 + PQ);
     // a round's rows travel global memory -> registers (one round ahead, while the round before is being used) ->
     // LDS; K as stored, V from its transposed copy: HD rows of PKEYS slots per round
     constexpr int VCH = PKEYS / 8;                                  // 16-byte chunks of a head element's slots in a round
@@ -186,8 +192,8 @@ attn_prefill_k(PrefillArgs a) {
     // round (scalar work).  A chunk the round does not need reads the round's first chunk instead, so that every load
     // is issued without a branch and nothing is computed per round and lane but a comparison and a selection.
     constexpr bool K_EVEN = PTH % NCH == 0;                         // then task t's key is task 0's + t * PTH / NCH
-    const char* const k_origin = reinterpret_cast<const char*>(a.k + (size_t)row0 * a.k_stride + (size_t)kvh * HD);
-    const char* const v_origin = reinterpret_cast<const char*>(a.vt + (size_t)kvh * HD * a.vt_rows + vt_base_of(a.cu_rows, seq));
+    const char* const k_origin = reinterpret_cast<const char*>(a.k + (size_t)krow0 * a.k_stride + (size_t)kvh * HD);
+    const char* const v_origin = reinterpret_cast<const char*>(a.vt + (size_t)kvh * HD * a.vt_rows + vt_base_of(a.cu_keys, seq));
     const size_t k_row_bytes = (size_t)a.k_stride * sizeof(bf16_t), v_row_bytes = (size_t)a.vt_rows * sizeof(bf16_t);
     unsigned koff[K_EVEN ? 1 : KTASKS];
     int kkey[K_EVEN ? 1 : KTASKS];
@@ -331,7 +337,7 @@ attn_prefill_k(PrefillArgs a) {
         for (int dt = 0; dt < HD / 16; dt++) o[dt] = o[dt] + *reinterpret_cast<const f32x4*>(theirs + dt * 4) * aj;
     }
     const float inv = 1.f / l;
-    bf16_t* orow = a.out + ((size_t)(row0 + qpos) * a.H + h) * HD;
+    bf16_t* orow = a.out + ((size_t)(row0 + qpos - qofs) * a.H + h) * HD;
 #pragma unroll
     for (int dt = 0; dt < HD / 16; dt++) {
         ushort4 pk;
@@ -354,28 +360,33 @@ static int prefill_launch(const PrefillArgs& a, int max_count, int H, int n_seq,
     return 0;
 }
 
-// elements of the transposed copy of V the prefill kernel needs as workspace
-extern "C" long tp_attn_prefill_workspace_elems(int M, int KV, int n_seq) {
-    return (long)KV * HD * ((long)M + (long)BKV * n_seq + BKV);
+// elements of the transposed copy of V the prefill kernel needs as workspace (Mk: rows of keys)
+extern "C" long tp_attn_prefill_workspace_elems(int Mk, int KV, int n_seq) {
+    return (long)KV * HD * ((long)Mk + (long)BKV * n_seq + BKV);
 }
 
+// q: M rows of queries, sequence s's at cu_rows[s] ..; k, v: Mk rows of keys and values, sequence s's at
+// cu_keys[s] .. (null: the queries' own rows, cu_rows); a sequence's queries are its last positions.
 extern "C" int tp_attn_prefill(const void* q, long q_stride, const void* k, long k_stride, const void* v, long v_stride,
                                int M, int H, int KV, const int* cu_rows, int n_seq, int max_count,
+                               const int* cu_keys, int Mk, int max_keys,
                                float scale, float cap, int window, void* out, void* workspace, void* stream) {
     TP_REQUIRE(M > 0 && H > 0 && KV > 0 && n_seq > 0 && max_count > 0, "attention prefill: empty shape");
     TP_REQUIRE(H % KV == 0, "attention: %d query heads are no multiple of %d kv heads", H, KV);
+    if (!cu_keys) { cu_keys = cu_rows; Mk = M; max_keys = max_count; }
+    TP_REQUIRE(Mk >= M && max_keys >= max_count, "attention prefill: %d keys (at most %d a sequence) for %d queries (at most %d)", Mk, max_keys, M, max_count);
     TP_REQUIRE(q_stride % 8 == 0 && k_stride % 8 == 0 && v_stride % 8 == 0 && (uintptr_t)q % 16 == 0 &&
                (uintptr_t)k % 16 == 0 && (uintptr_t)v % 16 == 0, "attention prefill: rows must be 16-byte aligned");
     TP_REQUIRE(n_seq <= 65535 && (long)tp_cdiv(max_count, 32) * H < (1L << 31), "attention prefill: %d heads / %d sequences exceed one launch", H, n_seq);
     TP_REQUIRE(workspace && (uintptr_t)workspace % 16 == 0, "attention prefill: needs its 16-byte aligned workspace");
-    TP_REQUIRE(k_stride < (1L << 22) && (long)HD * ((long)M + (long)BKV * n_seq + BKV) < (1L << 30),
-               "attention prefill: %d rows of stride %ld exceed the kernel's 32-bit offsets", M, k_stride);
+    TP_REQUIRE(k_stride < (1L << 22) && (long)HD * ((long)Mk + (long)BKV * n_seq + BKV) < (1L << 30),
+               "attention prefill: %d rows of stride %ld exceed the kernel's 32-bit offsets", Mk, k_stride);
     TP_REQUIRE(KV <= 65535, "attention prefill: %d kv heads exceed one launch", KV);
-    const long vt_rows = (long)M + (long)BKV * n_seq + BKV;         // every sequence's region is padded to whole groups
-    v_transpose_k<<<dim3(tp_cdiv(max_count, BKV), KV, n_seq), 256, 0, (hipStream_t)stream>>>(
-        (const bf16_t*)v, v_stride, KV, cu_rows, (bf16_t*)workspace, vt_rows);
+    const long vt_rows = (long)Mk + (long)BKV * n_seq + BKV;        // every sequence's region is padded to whole groups
+    v_transpose_k<<<dim3(tp_cdiv(max_keys, BKV), KV, n_seq), 256, 0, (hipStream_t)stream>>>(
+        (const bf16_t*)v, v_stride, KV, cu_keys, (bf16_t*)workspace, vt_rows);
     if (int rc = tp_check_launch("attention prefill (transpose of V)")) return rc;
-    PrefillArgs a{(const bf16_t*)q, q_stride, (const bf16_t*)k, k_stride, (const bf16_t*)v, v_stride, H, KV, cu_rows,
+    PrefillArgs a{(const bf16_t*)q, q_stride, (const bf16_t*)k, k_stride, (const bf16_t*)v, v_stride, H, KV, cu_rows, cu_keys,
                   scale, cap, window, (bf16_t*)out, (const bf16_t*)workspace, vt_rows};
     // 64 queries a block stage each key once per 64 queries; 32 a block make twice the blocks, for grids that would
     // not give every CU a block of 64 (measured, 8 heads of 256: 26 against 30 us at 512 tokens, 75 against 84 at

@@ -1,11 +1,15 @@
 """The geometry of one step: which rows belong to which sequence at which position.
 
 A step runs M rows packed without padding: sequence i brings counts[i] tokens at
-positions start[i] .. start[i] + counts[i] - 1.  Either every sequence starts
-(start 0, whole prompts: "prefill") or every sequence goes on by one token
-("decode").  The reference's step is one token of one sequence
-(runtime/src/lib.rs:4553); its only multi-token step takes consecutive positions
-of one sequence (runtime/src/lib.rs:845-869).
+positions start[i] .. start[i] + counts[i] - 1, start[i] being what the cache holds
+of it.  Any mix is a step: sequences that start, sequences that go on by one token,
+sequences that go on by several.  The engine names three shapes so that parts can
+pick their kernels: "decode" (every sequence brings one token), "prefill" (every
+sequence starts at its first token) and "extend" (anything else: a mixer then sees
+the cached positions before `start` as well as the step's own rows).  The
+reference's step is one token of one sequence (runtime/src/lib.rs:4553); its
+multi-token step takes M consecutive positions of one sequence from any position
+(runtime/src/lib.rs:845-869).
 """
 import numpy as np
 
@@ -23,12 +27,27 @@ def classify(counts, starts):
         return "decode"
     if all(s == 0 for s in starts):
         return "prefill"
-    raise StepError(
-        "a step either starts every sequence at its first token or continues every sequence by one token; "
-        f"found counts {list(counts)} at lengths {list(starts)}")
+    return "extend"
 
 
-def step_arrays(cache, slots, counts, starts, want_rows, table_widths=None):
+class KeyGeometry:
+    """Where a sequence's visible keys lie when a step gathers them into one buffer per cache group: the cached
+    positions prefix_lo[i] .. start[i] - 1 (all of them, or the last window - 1), then the step's own rows.
+    Sequence i's keys are rows cu_keys[i] .. cu_keys[i + 1] - 1, position t in row key_row0[i] + t."""
+
+    def __init__(self, starts, counts, window):
+        starts, counts = np.asarray(starts, dtype=np.int64), np.asarray(counts, dtype=np.int64)
+        self.prefix_lo = np.maximum(0, starts - (window - 1)) if window else np.zeros_like(starts)
+        keys = starts - self.prefix_lo + counts
+        self.cu_keys = np.zeros(len(starts) + 1, dtype=np.int64)
+        np.cumsum(keys, out=self.cu_keys[1:])
+        self.key_row0 = self.cu_keys[:-1] - self.prefix_lo
+        self.total_keys = int(self.cu_keys[-1])
+        self.max_keys = int(keys.max())
+        self.max_prefix = int((starts - self.prefix_lo).max())
+
+
+def step_arrays(cache, slots, counts, starts, want_rows, table_widths=None, key_geometry=()):
     """The step's geometry as int32 arrays, in the order StepContext slices them."""
     n, m = len(slots), int(sum(counts))
     cu = np.zeros(n + 1, dtype=np.int64)
@@ -45,6 +64,8 @@ def step_arrays(cache, slots, counts, starts, want_rows, table_widths=None):
         t = cache.page_table(gi, slots, None if table_widths is None else table_widths[gi])
         shapes.append(t.shape)
         parts.append(t.reshape(-1))
+    for g in key_geometry:
+        parts.extend([g.cu_keys, g.key_row0, g.prefix_lo])
     flat = np.concatenate([np.asarray(p, dtype=np.int32).reshape(-1) for p in parts])
     return flat, shapes
 
@@ -104,8 +125,11 @@ class StepContext:
         self._shared = set()            # entries whose step keys/values a later entry reads
         self._step_kv = {}
         n, m = self.n_seq, self.n_rows
+        self.key_geometry = []
+        if self.mode == "extend":
+            self.key_geometry = [KeyGeometry(self.starts, self.counts, g.spec.window) for g in cache.kv_groups]
         flat, shapes = step_arrays(cache, self.slots, self.counts, self.starts, want_rows,
-                                   static.table_widths if static is not None else None)
+                                   static.table_widths if static is not None else None, self.key_geometry)
         if static is not None:
             static.fill(flat)
             dev = static.device_buffer
@@ -127,9 +151,15 @@ class StepContext:
         self.identity_want = list(want_rows) == list(range(m))
         self.want_rows = take(self.n_want)
         self._tables = [take(int(np.prod(sh))).reshape(sh) for sh in shapes]
+        for g in self.key_geometry:          # the same numbers on the device
+            g.cu_keys_dev, g.key_row0_dev, g.prefix_lo_dev = take(n + 1), take(n), take(n)
 
     def page_table(self, group_index):
         return self._tables[group_index]
+
+    def keys_of(self, group_index):
+        """The KeyGeometry of a cache group in an "extend" step (host arrays, and `*_dev` int32 on the device)."""
+        return self.key_geometry[group_index]
 
     def max_keys(self, site):
         """Most keys any sequence of this step can see at this cache site (a host number, for launch geometry).
@@ -144,6 +174,7 @@ class StepContext:
         self._shared = set(entries)
 
     def offer_step_kv(self, k, v):
+        """k, v: the rows this step's attention reads (the step's own, or in an "extend" step the gathered ones)."""
         if self.entry in self._shared:
             self._step_kv[self.entry] = (k, v)
 

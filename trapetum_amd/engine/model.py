@@ -139,7 +139,7 @@ class Model:
             if s not in cache.book.length:
                 raise StepError(f"cache slot {s} is not in use")
         starts = [cache.length(s) for s in slots]
-        classify(counts, starts)                 # before the cache changes
+        classify(counts, starts)                 # refuses an empty step, before the cache changes
         cache.check_grow(slots, counts)
         for s, c in zip(slots, counts):
             cache.grow(s, c)

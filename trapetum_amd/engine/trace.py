@@ -6,7 +6,8 @@ file (runtime/src/bin/generate.rs:45-96).
 
 Input, one JSON object per line:
     {"step": 0, "entries": [{"id": "a", "tokens": [5, 17, 3], "want": [0, 2]}], "end": []}
-The requests of a step either all start or all continue by one token.  For a step with wanted places the
+A step may bring any number of tokens for each of its requests, whether they start or go on, and a request may
+join after others have started.  For a step with wanted places the
 logits go to <out>/<step>.f32 as little-endian float32 [wanted, vocab], in the order of entries and of want.
 After every step "done <step>" is printed and flushed.
 """

@@ -18,7 +18,9 @@ _CORE_SIGS = {
     "tp_rms_norm": [_P, _I, _P, _F, _P, _I, _I, _I, _P],
     "tp_add_rms_norm": [_P, _P, _I, _I, _L, _P, _F, _P, _F, _P, _I, _I, _I, _P],
     "tp_gather_rows": [_P, _P, _P, _I, _I, _I, _P],
-    "tp_rope_kv_write": [_P, _L, _P, _L, _P, _L, _I, _I, _I, _I, _I, _P, _I, _P, _P, _P, _P, _I, _P, _P, _I, _I, _P],
+    "tp_rope_kv_write": [_P, _L, _P, _L, _P, _L, _I, _I, _I, _I, _I, _P, _I, _P, _P, _P, _P, _I, _P, _P, _I, _I,
+                         _P, _P, _L, _P, _P],
+    "tp_gather_kv_prefix": [_P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P, _P, _P, _I, _P, _P, _L, _P],
     "tp_gated_act": [_P, _P, _I, _I, _I, _P],
     "tp_linear": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P, _L, _I, _I, _P],
     "tp_linear_workspace_bytes": [_I, _I, _I, _I, _I, _I, _I, _I, _I],
@@ -31,7 +33,7 @@ _CORE_SIGS = {
     "tp_sample_workspace_bytes": [_I, _I],
 }
 _ATTN_SIGS = {
-    "tp_attn_prefill": [_P, _L, _P, _L, _P, _L, _I, _I, _I, _P, _I, _I, _F, _F, _I, _P, _P, _P],
+    "tp_attn_prefill": [_P, _L, _P, _L, _P, _L, _I, _I, _I, _P, _I, _I, _P, _I, _I, _F, _F, _I, _P, _P, _P],
     "tp_attn_prefill_workspace_elems": [_I, _I, _I],
     "tp_attn_decode": [_P, _L, _I, _I, _I, _P, _P, _I, _P, _P, _I, _I, _F, _F, _I, _P, _P, _I, _P],
     "tp_attn_decode_workspace_floats": [_I, _I, _I],
@@ -196,7 +198,9 @@ class HipOps:
         return out
 
     def rope_kv_write(self, q, k, v, H, KV, hd, inv_freq, rotary_dim, row_seq, row_pos, new_len, table,
-                      k_pool, v_pool, rows_cap):
+                      k_pool, v_pool, rows_cap, gathered=None):
+        """Rotate q and k in place and write k, v into the cache.  gathered = (gk, gv, key_row0): the step's rows
+        also go into the buffers that `gather_kv_prefix` began, position t of sequence s into row key_row0[s] + t."""
         self._dev(q, k, v, inv_freq, row_seq, row_pos, new_len, table, k_pool, v_pool)
         m = q.shape[0]
         qs = self._rows(q, "rope_kv_write q")
@@ -221,11 +225,44 @@ class HipOps:
                 raise KernelError("rope_kv_write: the page table must be contiguous int32 [sequences, pages]")
             page, table_w = k_pool.shape[2], table.shape[1]
             kp, vp = k.data_ptr(), v.data_ptr()
+        gk = gv = row0 = None
+        g_stride = 0
+        if gathered is not None:
+            gk, gv, row0 = gathered
+            self._dev(gk, gv, row0)
+            if k is None or gk.dtype != q.dtype or gv.dtype != q.dtype or gk.shape != gv.shape or gk.dim() != 2 \
+                    or gk.shape[1] != KV * hd or not gk.is_contiguous() or not gv.is_contiguous():
+                raise KernelError("rope_kv_write: the gathered buffers must be contiguous [keys, kv_heads * head_dim] of q's dtype")
+            if row0.dtype != torch.int32 or row0.numel() != new_len.numel():
+                raise KernelError("rope_kv_write: one int32 row origin per sequence")
+            g_stride = gk.stride(0)
         self._call(self.lib, "tp_rope_kv_write", q.data_ptr(), qs, kp or None, ks, vp or None, vs, _code(q.dtype), m, H, KV, hd,
                    inv_freq.data_ptr() if rotary_dim else None, rotary_dim, row_seq.data_ptr(), row_pos.data_ptr(),
                    new_len.data_ptr(), table.data_ptr() if k is not None else None, table_w,
                    k_pool.data_ptr() if k is not None else None, v_pool.data_ptr() if k is not None else None,
-                   page, rows_cap, self._stream())
+                   page, rows_cap, gk.data_ptr() if gk is not None else None, gv.data_ptr() if gv is not None else None,
+                   g_stride, row0.data_ptr() if row0 is not None else None, self._stream())
+
+    def gather_kv_prefix(self, table, k_pool, v_pool, rows_cap, cu_rows, keys):
+        """Buffers gk, gv [keys.total_keys, kv_heads * head_dim] with every sequence's cached positions
+        keys.prefix_lo[s] .. start[s] - 1 copied out of the cache (sequence s's position t in row keys.key_row0[s] + t);
+        the rows of the step itself are left for `rope_kv_write(..., gathered=)`.  keys: the step's KeyGeometry."""
+        self._dev(table, k_pool, v_pool, cu_rows, keys.cu_keys_dev, keys.prefix_lo_dev)
+        n = table.shape[0]
+        if k_pool.dim() != 4 or v_pool.shape != k_pool.shape or not k_pool.is_contiguous() or not v_pool.is_contiguous():
+            raise KernelError("gather_kv_prefix: cache pools must be contiguous [pages, kv_heads, page, head_dim]")
+        if table.dtype != torch.int32 or table.dim() != 2 or not table.is_contiguous():
+            raise KernelError("gather_kv_prefix: the page table must be contiguous int32 [sequences, pages]")
+        for t, size in ((cu_rows, n + 1), (keys.cu_keys_dev, n + 1), (keys.prefix_lo_dev, n)):
+            if t.dtype != torch.int32 or t.numel() != size:
+                raise KernelError("gather_kv_prefix: the step's geometry must be int32 arrays over its sequences")
+        _, KV, page, hd = k_pool.shape
+        gk = torch.empty((keys.total_keys, KV * hd), dtype=k_pool.dtype, device=self.device)
+        gv = torch.empty_like(gk)
+        self._call(self.lib, "tp_gather_kv_prefix", k_pool.data_ptr(), v_pool.data_ptr(), _code(k_pool.dtype), table.data_ptr(),
+                   table.shape[1], page, rows_cap, KV, hd, n, cu_rows.data_ptr(), keys.cu_keys_dev.data_ptr(),
+                   keys.prefix_lo_dev.data_ptr(), int(keys.max_prefix), gk.data_ptr(), gv.data_ptr(), gk.stride(0), self._stream())
+        return gk, gv
 
     # ---- matrix products -----------------------------------------------------------------------------
     def _linear(self, x, w, out_dtype, epilogue, cap, units, defer=False):
@@ -272,29 +309,38 @@ class HipOps:
                 and H // KV <= 16 and _build.ATTN_SOURCE in _build.os.listdir(_build.CSRC))
 
     def attention_prefill(self, q, k, v, H, KV, hd, cu_rows, max_count, scale, softcap, window, out_dtype,
-                          row_seq=None, row_pos=None):
+                          row_seq=None, row_pos=None, keys=None):
+        """Causal attention of the step's queries over rows of keys and values: the step's own (every sequence
+        starts: row_pos counts from 0), or with `keys` (a KeyGeometry) the gathered buffers, in which sequence s's
+        position t is row keys.key_row0[s] + t and row_pos holds absolute positions."""
         self._dev(q, k, v, cu_rows)
         m = q.shape[0]
+        mk = m if keys is None else keys.total_keys
         qs, ks, vs = self._rows(q, "attention q"), self._rows(k, "attention k"), self._rows(v, "attention v")
-        if q.shape[1] != H * hd or k.shape != (m, KV * hd) or v.shape != (m, KV * hd):
-            raise KernelError("attention_prefill: q, k, v must be [rows, heads * head_dim]")
+        if q.shape[1] != H * hd or k.shape != (mk, KV * hd) or v.shape != (mk, KV * hd):
+            raise KernelError("attention_prefill: q must be [rows, heads * head_dim], k and v [keys, kv_heads * head_dim]")
         if not (q.dtype == k.dtype == v.dtype == out_dtype):
             raise KernelError("attention_prefill: q, k, v and the output share one dtype")
         n_seq = cu_rows.numel() - 1
         out = torch.empty((m, H * hd), dtype=out_dtype, device=self.device)
         if self._fast_attention(q.dtype, H, KV, hd):
             lib = self.attn_lib(hd)
-            ws = torch.empty(lib.tp_attn_prefill_workspace_elems(m, KV, n_seq), dtype=torch.bfloat16, device=self.device)
+            ws = torch.empty(lib.tp_attn_prefill_workspace_elems(mk, KV, n_seq), dtype=torch.bfloat16, device=self.device)
             self._call(lib, "tp_attn_prefill", q.data_ptr(), qs, k.data_ptr(), ks, v.data_ptr(), vs,
-                       m, H, KV, cu_rows.data_ptr(), n_seq, int(max_count), float(scale), float(softcap), int(window),
-                       out.data_ptr(), ws.data_ptr(), self._stream())
+                       m, H, KV, cu_rows.data_ptr(), n_seq, int(max_count),
+                       keys.cu_keys_dev.data_ptr() if keys is not None else None, mk,
+                       int(keys.max_keys) if keys is not None else int(max_count),
+                       float(scale), float(softcap), int(window), out.data_ptr(), ws.data_ptr(), self._stream())
             return out
+        if keys is not None and (row_seq is None or row_pos is None):
+            raise KernelError("attention_prefill: gathered keys need every row's sequence and position")
         if row_seq is None:
             counts = (cu_rows[1:] - cu_rows[:-1]).long()
             row_seq = torch.repeat_interleave(torch.arange(n_seq, device=self.device, dtype=torch.int32), counts)
             row_pos = (torch.arange(m, device=self.device, dtype=torch.int32) - cu_rows[:-1][row_seq.long()]).to(torch.int32)
+        key_rows = cu_rows if keys is None else keys.key_row0_dev       # where a sequence's position 0 would lie
         self._call(self.lib, "tp_attn_simple_prefill", q.data_ptr(), qs, k.data_ptr(), ks, v.data_ptr(), vs, _code(q.dtype),
-                   m, H, KV, hd, cu_rows.data_ptr(), row_seq.data_ptr(), row_pos.data_ptr(), float(scale), float(softcap),
+                   m, H, KV, hd, key_rows.data_ptr(), row_seq.data_ptr(), row_pos.data_ptr(), float(scale), float(softcap),
                    int(window), out.data_ptr(), self._stream())
         return out
 

@@ -13,7 +13,9 @@ The three projections are one product over the concatenated weight.  A run that
 reads another run's cache projects and rotates its queries only.  In a decode step
 rotation, cache write and attention are one kernel launch where the kernel library
 has one for the geometry (`ops.fuses_decode_step`); the order of the arithmetic is
-the same.
+the same.  A step that continues sequences by several tokens, or mixes starting and running sequences, attends
+over the cached positions its queries still see plus its own rows (the reference's multi-token step does the
+same from any position: runtime/src/lib.rs:676-720, runtime/cuda/codebook_gemv.cu:410-440).
 """
 from ..cache.store import KVSpec
 from ..models.spec import TensorSpec
@@ -58,6 +60,8 @@ class Attention(Mixer):
         H, KV, hd = self.num_heads, self.num_kv_heads, self.head_dim
         Q, KVD = H * hd, KV * hd
         owns_cache = ctx.cache_owner == ctx.entry
+        if site.spec.window is not None and not 0 < self.window <= site.spec.window:
+            raise ValueError(f"this attention sees {self.window or 'all'} keys back, the cache it reads keeps {site.spec.window}")
         table = ctx.page_table(site.group_index)
         rows_cap = site.rows_cap or 0
         if ctx.mode == "decode" and ops.fuses_decode_step(ctx.dtype, H, KV, hd, site.k):
@@ -72,20 +76,31 @@ class Attention(Mixer):
             q, k, v = qkv[:, :Q], qkv[:, Q:Q + KVD], qkv[:, Q + KVD:]
         else:
             q, k, v = ops.linear(x, self.w_qkv[:Q], ctx.dtype), None, None
+        keys = gathered = None
+        if ctx.mode == "extend":
+            # Sequences go on by several tokens (or some start while others go on): the queries see cached positions
+            # and the step's own rows.  The cached ones are copied out first, because the step's rows may take their
+            # places in a window's ring; the step's rows join them in the same buffers as they are rotated.
+            keys = ctx.keys_of(site.group_index)
+            if owns_cache:
+                gk, gv = ops.gather_kv_prefix(table, site.k, site.v, rows_cap, ctx.cu_rows, keys)
+                gathered = (gk, gv, keys.key_row0_dev)
         ops.rope_kv_write(q, k, v, H, KV, hd, self.inv_freq, self.position.rotary_dim,
-                          ctx.row_seq, ctx.row_pos, ctx.new_len, table, site.k, site.v, rows_cap)
-        if ctx.mode == "prefill":
+                          ctx.row_seq, ctx.row_pos, ctx.new_len, table, site.k, site.v, rows_cap, gathered=gathered)
+        if ctx.mode == "decode":
+            out = ops.attention_decode(q, H, KV, hd, ctx.new_len, table, site.k, site.v, rows_cap,
+                                       self.query_scale, self.softcap, self.window, ctx.dtype,
+                                       max_keys=ctx.max_keys(site))
+        else:
+            if gathered is not None:
+                k, v = gathered[0], gathered[1]
             if owns_cache:
                 ctx.offer_step_kv(k, v)
             else:
                 k, v = ctx.step_kv_of(ctx.cache_owner)
             out = ops.attention_prefill(q, k, v, H, KV, hd, ctx.cu_rows, ctx.max_count,
                                         self.query_scale, self.softcap, self.window, ctx.dtype,
-                                        row_seq=ctx.row_seq, row_pos=ctx.row_pos)
-        else:
-            out = ops.attention_decode(q, H, KV, hd, ctx.new_len, table, site.k, site.v, rows_cap,
-                                       self.query_scale, self.softcap, self.window, ctx.dtype,
-                                       max_keys=ctx.max_keys(site))
+                                        row_seq=ctx.row_seq, row_pos=ctx.row_pos, keys=keys)
         return ops.linear(out, self.w_o, ctx.dtype, defer=True)
 
 
