@@ -142,7 +142,11 @@ def attention_block(x, positions, W, p, cfg, window, rnd):
 
 
 def layer_window(cfg, layer):
-    """Even layers are local (window), odd layers global."""
+    """Even layers are local (window), odd layers global, unless config.json lists `layer_types`
+    (the reference models no window: runtime/src/lib.rs:4455)."""
+    kinds = cfg.get("layer_types")
+    if kinds:
+        return cfg["sliding_window"] if kinds[layer] == "sliding_attention" else None
     return cfg["sliding_window"] if layer % 2 == 0 else None
 
 

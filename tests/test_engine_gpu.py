@@ -119,3 +119,96 @@ def test_portions_and_joining_requests(setup, page_size):
         assert cache.live_slots() == []
         for rid in requests:
             assert rel_l2(torch.from_numpy(got[rid]), ref[rid]) < tol, rid
+
+
+class _Tensors:
+    """Weights held in memory, for `load_into`."""
+
+    def __init__(self, tensors):
+        self.tensors = tensors
+
+    def names(self):
+        return list(self.tensors)
+
+    def shape(self, name):
+        return tuple(self.tensors[name].shape)
+
+    def dtype(self, name):
+        return self.tensors[name].dtype
+
+    def tensor(self, name):
+        return self.tensors[name]
+
+
+def _model_of(folder, dtype, tensors=None):
+    from trapetum_amd.engine.model import Model
+    from trapetum_amd.engine.runtime import Runtime
+    from trapetum_amd.registry import config_from_folder
+    from trapetum_amd.weights import WeightFolder, load_folder, load_into
+    arch, cfg = config_from_folder(folder)
+    model = Model(arch.build_spec(cfg), Runtime(dtype=dtype, device="cuda:0"))
+    if tensors is None:
+        load_folder(model, folder)
+    else:
+        load_into(model, _Tensors(tensors))
+    return model, cfg
+
+
+def _whole(model, toks):
+    cache = model.new_cache(max_tokens=128, page_size=16)
+    s = cache.acquire()
+    return model.step(cache, [s], toks, counts=[len(toks)], want=list(range(len(toks)))).double().cpu()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_layer_0_is_local_and_layer_types_overrides(tmp_path, dtype):
+    """A model of layer 0 alone (tiny B, window 16): a changed token 0 leaves the logits at positions >= 16 untouched,
+    bit for bit, because an even layer is local; `layer_types` naming it full_attention flips that.  Fails when the
+    engine takes odd layers for the local ones or ignores `layer_types`."""
+    folder = make_folder(tmp_path, "B", name="one_layer", num_hidden_layers=1)
+    model, cfg = _model_of(folder, dtype)
+    toks = random_tokens(40, cfg.vocab_size, 5)
+    other = [(toks[0] + 1) % cfg.vocab_size] + toks[1:]
+    a, b = _whole(model, toks), _whole(model, other)
+    assert torch.equal(a[16:], b[16:]) and not torch.equal(a[15], b[15])
+    pcfg, pw = plain.read_folder(folder)
+    assert rel_l2(a, plain.forward(pcfg, pw, toks)) < TOL[dtype]
+    folder = make_folder(tmp_path, "B", name="one_full_layer", num_hidden_layers=1, layer_types=["full_attention"])
+    model, cfg = _model_of(folder, dtype)
+    a, b = _whole(model, toks), _whole(model, other)
+    assert not torch.equal(a[39], b[39])
+    pcfg, pw = plain.read_folder(folder)
+    assert pcfg["layer_types"] == ["full_attention"] and rel_l2(a, plain.forward(pcfg, pw, toks)) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_no_layers_oracle_and_sandwich_identity(tmp_path, dtype):
+    """Without layers the logits are norm(E[tok] * sqrt(D)) @ E^T (the lookup is scaled, the head is not), and with
+    post-norm weights of -1 (a gain of 0) every layer adds nothing, so the same holds with layers.  Fails when a
+    post-norm is applied to the sub-layer's input instead of its output, or the head uses the scaled table."""
+    import math
+    folder = make_folder(tmp_path, "B", name="no_layers", num_hidden_layers=0)
+    model, cfg = _model_of(folder, dtype)
+    pcfg, pw = plain.read_folder(folder)
+    toks = random_tokens(7, cfg.vocab_size, 1)
+    e = pw["model.embed_tokens.weight"]
+    x = e[toks] * math.sqrt(cfg.hidden_size)
+    n = x / torch.sqrt((x * x).mean(-1, keepdim=True) + cfg.rms_norm_eps) * (1 + pw["model.norm.weight"])
+    oracle = n @ e.T
+    assert rel_l2(_whole(model, toks), oracle) < TOL[dtype]
+    from trapetum_amd.weights import WeightFolder
+    folder = make_folder(tmp_path, "B")
+    src = WeightFolder(folder)
+    tensors = {name: src.tensor(name).clone() for name in src.names()}
+    src.close()
+    for name in tensors:
+        if "post_attention_layernorm" in name or "post_feedforward_layernorm" in name:
+            tensors[name] = -torch.ones_like(tensors[name])
+    model, cfg = _model_of(folder, dtype, tensors)
+    pcfg, pw = plain.read_folder(folder)                     # the same embedding and final norm: the same oracle
+    e = pw["model.embed_tokens.weight"]
+    x = e[toks] * math.sqrt(cfg.hidden_size)
+    n = x / torch.sqrt((x * x).mean(-1, keepdim=True) + cfg.rms_norm_eps) * (1 + pw["model.norm.weight"])
+    assert rel_l2(_whole(model, toks), n @ e.T) < TOL[dtype]
+    model, cfg = _model_of(folder, dtype)
+    assert rel_l2(_whole(model, toks), n @ e.T) > 10 * TOL[dtype]

@@ -57,7 +57,6 @@ def test_norm(rt):
     norm = build_part("norm", ("rms_norm", {"size": 88, "eps": 1e-4, "weight_offset": 1.0}))
     w = bound(norm, rt, {"weight": rnd(88, seed=1, scale=0.3)})
     x = rnd(7, 88, seed=2, scale=2.0)
-    ctx = OnePartContext(rt, None).step([], []) if False else None
     got = norm.forward(type("C", (), {"ops": rt.ops, "dtype": rt.dtype})(), x.to(DEV))
     assert rel_l2(got, plain.rms_norm(x.double(), w["weight"], 1e-4)) < TOL[str(rt.dtype).split(".")[1]]
     plain_norm = build_part("norm", ("rms_norm", {"size": 88, "eps": 1e-4}))        # without the offset: gain = w
@@ -157,6 +156,52 @@ def test_window_edge_shows(rt):
     s = one2.cache.acquire()
     rows = [rt.ops.rows(mixer.forward(one2.step([s], [1]), act(rt, x[i:i + 1]), one2.cache.site(0)), rt.dtype) for i in range(20)]
     assert rel_l2(torch.cat(rows), ref) < tol
+
+
+def test_cap_comes_after_the_scale(rt):
+    """Dots of +1e6 and -1e6 with a scale of 1/4 and a cap of 3: the probabilities are softmax([+3, -3]) if the cap is
+    applied to the scaled score (runtime/cuda/codebook_gemv.cu:254-255) and softmax([+3/4, -3/4]) if the scale came
+    after the cap; random weights cannot tell the two apart, because tanh is linear for their small scores.  Whole
+    prompt and token by token; fails when a kernel multiplies by the scale after the cap."""
+    tol = 3e-6 if rt.dtype == torch.float32 else 1.5e-2
+    mixer = build_part("mixer", ("attention", dict(ATT, softcap=3.0, query_scale=0.25, window=None, position=("none", {}))))
+    w = bound(mixer, rt, {"q_proj.weight": torch.eye(192, 88), "k_proj.weight": -torch.eye(64, 88),
+                          "v_proj.weight": rnd(64, 88, seed=15), "o_proj.weight": torch.eye(88, 192)})
+    x = torch.zeros(2, 88)
+    x[0, 0], x[1, 0] = -1e3, 1e3                           # keys +1e3 and -1e3 on element 0, the query at position 1 +1e3
+    x[:, 40:] = rnd(2, 48, seed=16)                         # what the values are made of
+    x = x.to(torch.bfloat16)
+    v = (x.double() @ w["v_proj.weight"].T)[:, :32]         # kv head 0, which query head 0 reads
+    p = torch.softmax(torch.tensor([3.0, -3.0], dtype=torch.float64), 0)
+    want = p[0] * v[0] + p[1] * v[1]
+    wrong = torch.softmax(torch.tensor([0.75, -0.75], dtype=torch.float64), 0)
+    assert rel_l2(wrong[0] * v[0] + wrong[1] * v[1], want) > 0.1
+    one = OnePartContext(rt, mixer.cache_spec())
+    s = one.cache.acquire()
+    got = rt.ops.rows(mixer.forward(one.step([s], [2]), act(rt, x), one.cache.site(0)), rt.dtype)
+    assert rel_l2(got[1, :32], want) < tol
+    one = OnePartContext(rt, mixer.cache_spec())
+    s = one.cache.acquire()
+    rows = [rt.ops.rows(mixer.forward(one.step([s], [1]), act(rt, x[i:i + 1]), one.cache.site(0)), rt.dtype) for i in range(2)]
+    assert rel_l2(rows[1][0, :32], want) < tol
+
+
+@pytest.mark.parametrize("m", [1, 8, 200])
+def test_the_gate_is_what_the_activation_is_applied_to(rt, m):
+    """gate = -20 and up = +5 give gelu_tanh(-20) * 5 = 0; with the two swapped the result is gelu_tanh(5) * -20 = -100
+    (runtime/cuda/codebook_gemv.cu:531-537, runtime/src/lib.rs:4511-4513).  One, a few and many rows run on different
+    product kernels; fails when a gated epilogue activates the up half."""
+    ff = build_part("feed_forward", ("gated_mlp", {"hidden_size": 16, "intermediate_size": 16, "activation": "gelu_tanh"}))
+    gate, up = torch.zeros(16, 16), torch.zeros(16, 16)
+    gate[:, 0], up[:, 0] = -20.0, 5.0
+    bound(ff, rt, {"gate_proj.weight": gate, "up_proj.weight": up, "down_proj.weight": torch.eye(16)})
+    x = torch.zeros(m, 16)
+    x[:, 0] = 1.0
+    got = rt.ops.rows(ff.forward(type("C", (), {"ops": rt.ops, "dtype": rt.dtype})(), act(rt, x)), rt.dtype)
+    assert float(got.float().abs().max()) < 1e-3
+    bound(ff, rt, {"gate_proj.weight": up, "up_proj.weight": gate, "down_proj.weight": torch.eye(16)})
+    got = rt.ops.rows(ff.forward(type("C", (), {"ops": rt.ops, "dtype": rt.dtype})(), act(rt, x)), rt.dtype)
+    assert float((got.float() + 100.0).abs().max()) < 0.5
 
 
 def test_sandwich_block(rt):

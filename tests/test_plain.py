@@ -98,6 +98,37 @@ def test_attention_grouping_scale_cap_window():
     assert float(plain.softcap(torch.tensor([-3.0], dtype=D), 7.0)) == -float(plain.softcap(torch.tensor([3.0], dtype=D), 7.0))
 
 
+def saturating_case():
+    """Two keys whose dots with the query at position 1 are +1e6 and -1e6: the capped scores are +cap and -cap
+    whatever the scale, if the cap comes after the scale."""
+    q, k = torch.zeros(2, 1, 4, dtype=D), torch.zeros(2, 1, 4, dtype=D)
+    q[1, 0, 0], k[0, 0, 0], k[1, 0, 0] = 1e3, 1e3, -1e3
+    v = rnd(2, 1, 4, seed=30)
+    return q, k, v
+
+
+def test_cap_comes_after_the_scale():
+    """score = dot * scale, then cap * tanh(score / cap) (runtime/cuda/codebook_gemv.cu:254-255).  With saturating dots and
+    a scale of 1/4 the probabilities are softmax([+cap, -cap]); capping first and scaling after gives
+    softmax([+cap/4, -cap/4]).  Fails when `softcap` in plain.attention moves before the multiplication by the scale."""
+    q, k, v = saturating_case()
+    got = plain.attention(q, k, v, 0.25, 3.0, None)[1, 0]
+    p = torch.softmax(torch.tensor([3.0, -3.0], dtype=D), 0)
+    assert torch.allclose(got, p[0] * v[0, 0] + p[1] * v[1, 0], atol=1e-12)
+    wrong = torch.softmax(torch.tensor([0.75, -0.75], dtype=D), 0)
+    assert not torch.allclose(got, wrong[0] * v[0, 0] + wrong[1] * v[1, 0], atol=1e-3)
+
+
+def test_the_gate_is_what_the_activation_is_applied_to():
+    """act = gelu_tanh(gate) * up (runtime/cuda/codebook_gemv.cu:531-537 with g = gate, u = up: runtime/src/lib.rs:4511-4513).
+    A gate of -20 with an up of +5 gives 0; the swap, gelu_tanh(5) * -20, gives -100.  Fails when the activation moves
+    to the up projection in plain.geglu."""
+    one = torch.ones(1, 1, dtype=D)
+    got = plain.geglu(one, -20.0 * one, 5.0 * one, one, lambda t: t)
+    assert abs(float(got)) < 1e-9
+    assert abs(float(plain.geglu(one, 5.0 * one, -20.0 * one, one, lambda t: t)) + 100.0) < 1e-3
+
+
 # ---- feed-forward, embedding, head, sandwich ---------------------------------------------------------------------
 def test_gelu_and_geglu():
     g = torch.linspace(-6, 6, 101, dtype=D)
@@ -156,6 +187,23 @@ def test_local_layers_forget_and_global_layers_do_not(folder_b):
     finally:
         plain.layer_window = plain_window
     assert torch.equal(a[3 * 15 + 1:], b[3 * 15 + 1:]) and not torch.allclose(a[30], b[30], atol=1e-12)
+
+
+def test_layer_0_is_local_and_layer_types_overrides(folder_b):
+    """A model of layer 0 alone (window 16): a changed token 0 leaves the logits at positions >= 16 untouched, because an
+    even layer is local; `layer_types` naming it full_attention flips that.  Fails when the parity in plain.layer_window
+    is swapped (layer 0 global), or when `layer_types` is ignored."""
+    cfg, w = plain.read_folder(folder_b)
+    one = dict(cfg, num_hidden_layers=1)
+    toks = random_tokens(40, cfg["vocab_size"], 5)
+    other = [(toks[0] + 1) % cfg["vocab_size"]] + toks[1:]
+    a, b = plain.forward(one, w, toks), plain.forward(one, w, other)
+    assert torch.equal(a[16:], b[16:]) and not torch.allclose(a[15], b[15], atol=1e-9)
+    full = dict(one, layer_types=["full_attention"])
+    a, b = plain.forward(full, w, toks), plain.forward(full, w, other)
+    assert not torch.allclose(a[39], b[39], atol=1e-9)
+    two = dict(cfg, num_hidden_layers=2, layer_types=["full_attention", "sliding_attention"])
+    assert not torch.allclose(plain.forward(two, w, toks)[39], plain.forward(dict(cfg, num_hidden_layers=2), w, toks)[39], atol=1e-9)
 
 
 # ---- token choice --------------------------------------------------------------------------------------------------

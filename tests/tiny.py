@@ -43,10 +43,11 @@ TINY_D_INIT = dict(seed=6, sigma=0.06, sigma_norm=0.2)
 CONFIGS = {"A": (TINY_A, TINY_A_INIT), "B": (TINY_B, TINY_B_INIT), "C": (TINY_C, TINY_C_INIT), "D": (TINY_D, TINY_D_INIT)}
 
 
-def make_folder(tmp_path, which):
+def make_folder(tmp_path, which, name=None, **overrides):
+    """A model folder of one of the tiny configurations; `overrides` replace config keys (folder `name` then)."""
     cfg_kw, init = CONFIGS[which]
-    cfg = Gemma2Config.from_kwargs(**cfg_kw)
-    folder = os.path.join(str(tmp_path), f"tiny_{which}")
+    cfg = Gemma2Config.from_kwargs(**dict(cfg_kw, **overrides))
+    folder = os.path.join(str(tmp_path), name or f"tiny_{which}")
     write_model_folder(cfg, folder, **init)
     return folder
 

@@ -40,10 +40,12 @@ class Gemma2Config(ModelConfig):
     layer_types: tuple = key("layer_types", "str_list", None, doc="per layer: sliding_attention or full_attention")
 
     def validate(self):
-        for name in ("num_hidden_layers", "hidden_size", "num_attention_heads", "num_key_value_heads",
+        for name in ("hidden_size", "num_attention_heads", "num_key_value_heads",
                      "head_dim", "intermediate_size", "vocab_size", "sliding_window"):
             if getattr(self, name) <= 0:
                 raise ConfigError(f"config key '{name}' must be positive, found {getattr(self, name)}")
+        if self.num_hidden_layers < 0:      # none at all is a model too: embedding, final norm, head
+            raise ConfigError(f"config key 'num_hidden_layers' must not be negative, found {self.num_hidden_layers}")
         if self.num_attention_heads % self.num_key_value_heads:
             raise ConfigError(
                 f"num_attention_heads ({self.num_attention_heads}) is no multiple of "
