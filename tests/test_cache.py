@@ -31,9 +31,13 @@ def test_groups_and_sites():
     local, glob = c.kv_groups
     assert local.entries == [0, 2] and glob.entries == [1]
     assert local.pages.rows_cap == 48 and glob.pages.rows_cap is None        # window 40 -> ring of 3 pages of 16
-    assert tuple(local.k_pool.shape) == (2, 32, 2, 16, 16)
+    # 4 slots with rings of 3 pages never hold more than 12 pages; the other group may hold all 32; one spare each
+    assert tuple(local.k_pool.shape) == (2, 12 + 1, 2, 16, 16) and tuple(glob.k_pool.shape) == (1, 32 + 1, 2, 16, 16)
+    assert local.spare_page == 12 and glob.spare_page == 32 and c.spare_slot == 4
     assert c.site(0).group_index == 0 and c.site(2).index_in_group == 1 and c.site(4) is None
-    assert tuple(c.site(3).state.shape) == (4, 3, 5)
+    assert tuple(c.site(3).state.shape) == (4 + 1, 3, 5)                      # one spare slot
+    t = c.page_table(0, [c.spare_slot], width=3)                              # the spare slot's row names the spare page
+    assert list(t[0]) == [12, -1, -1]
     wide = make(window=1000)                                                  # a window beyond the context keeps every row
     assert wide.kv_groups[0].pages.rows_cap is None
 
@@ -51,7 +55,7 @@ def test_pages_follow_lengths():
     with pytest.raises(CacheError, match="context overflow"):
         c.grow(s, 200)
     c.release(s)
-    assert c.tokens_held() == 0 and all(g.pages.pool.available() == 32 for g in c.kv_groups)
+    assert c.tokens_held() == 0 and [g.pages.pool.available() for g in c.kv_groups] == [12, 32]
     with pytest.raises(CacheError, match="twice"):
         c.release(s)
 

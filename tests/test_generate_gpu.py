@@ -50,9 +50,14 @@ def test_sampled_generation_equals_plain_sampler(folders, top_p, top_k):
             out.append(tok)
             seq.append(tok)
         assert got[i] == out, i
-    # each request alone gives what it gave in the batch
-    alone = engine.generate([prompts[2]], max_tokens=12, temperature=0.7, top_p=top_p, top_k=top_k, seed=7, stop_ids=())
-    assert alone[0] != [] and len(alone[0]) == 12
+    # each request alone, under the id it had in the batch, gives what it gave in the batch
+    for i in (2, 0):
+        alone = engine.generate([prompts[i]], max_tokens=12, temperature=0.7, top_p=top_p, top_k=top_k, seed=7,
+                                stop_ids=(), request_ids=[i])
+        assert alone[0] == got[i], i
+    # and under another id other tokens
+    assert engine.generate([prompts[2]], max_tokens=12, temperature=0.7, top_p=top_p, top_k=top_k, seed=7,
+                           stop_ids=(), request_ids=[5])[0] != got[2]
 
 
 @pytest.mark.parametrize("dtype,tol", [("float32", 1e-5), ("bfloat16", 2e-2)])
@@ -97,7 +102,7 @@ def test_graph_replays_equal_eager_steps(folders):
         torch.cuda.synchronize()
         assert torch.equal(a, b), step
         torch.randn(64, 64, device="cuda:0").sum().item()          # unrelated eager work between replays
-    # a smaller batch gets its own graph; the larger one still replays afterwards
+    # a smaller batch gets a graph of fewer rows
     graph_cache.release(gs.pop())
     eager_cache.release(es.pop())
     for step in range(12, 16):
@@ -126,23 +131,44 @@ def test_graphs_follow_a_sequence_across_their_length_bound(folders):
         a = model.step(eager_cache, es, step_toks).clone()
         b = graphed.step(gs, step_toks).clone()
         assert rel_l2(b, a) < 3e-3, step
-    assert len(graphed.by_batch) == 2
+    assert len(graphed.graphs) == 2 and graphed.captures == 2
 
 
-def test_decode_loop_with_and_without_graph(folders):
-    """The device-resident greedy loop: the graph that also picks the tokens gives the ids of eager steps and argmax."""
-    from .gpu_engine import load_gpu_model
-    from trapetum_amd.engine.decode_loop import DecodeLoop
-    model, cfg = load_gpu_model(folders["B"], "bfloat16")
-    prompts = [random_tokens(n, cfg.vocab_size, 70 + i) for i, n in enumerate((7, 19, 33))]
-    runs = []
+def test_a_shrinking_batch_with_and_without_graphs(folders):
+    """Eight requests that reach the context's end one after the other: the graphs' rows that stand for no sequence any
+    more, and the moves into graphs of fewer rows, change no token (greedy, and sampled inside the graph)."""
+    from trapetum_amd import load_model
+    pcfg, pw = plain.read_folder(folders["B"])
+    context, most = 48, 40
+    prompts = [random_tokens(n, pcfg["vocab_size"], 70 + i) for i, n in enumerate((12, 45, 27, 9, 42, 20, 38, 33))]
+    limits = [min(most, context + 1 - len(p)) for p in prompts]          # 37, 4, 22, 40, 7, 29, 11, 16 tokens
+    want = [plain.greedy_generate(pcfg, pw, p, n) for p, n in zip(prompts, limits)]
+    runs = {}
     for use_graph in (False, True):
-        cache = model.new_cache(max_tokens=1024, page_size=16)
-        loop = DecodeLoop(model, cache, use_graph=use_graph)
-        ids = [loop.start(prompts).cpu().tolist()]
-        for _ in range(20):
-            ids.append(loop.step().cpu().tolist())
-            torch.randn(32, 32, device="cuda:0").sum().item()       # unrelated eager work between replays
-        loop.finish()
-        runs.append(ids)
-    assert runs[0] == runs[1]
+        engine = load_model(folders["B"], dtype="float32", max_tokens_in_cache=2048, max_context=context, max_batch=8,
+                            use_graph=use_graph)
+        got = engine.generate(prompts, max_tokens=most, stop_ids=(), with_reasons=True)
+        runs[use_graph] = [g.tokens for g in got]
+        assert [g.reason for g in got] == ["context" if n < most else "length" for n in limits]
+        assert engine.cache.live_slots() == []
+        if use_graph:
+            assert {k[0] for k in engine.graphed.graphs} == {8, 4, 2, 1}    # the batch moved through smaller graphs
+        sampled = engine.generate(prompts, max_tokens=most, temperature=0.9, top_p=0.9, top_k=30, seed=3, stop_ids=())
+        runs[use_graph, "sampled"] = sampled
+    assert runs[True] == want and runs[False] == want
+    assert runs[True, "sampled"] == runs[False, "sampled"] and [len(t) for t in runs[True, "sampled"]] == limits
+
+
+def test_graphs_are_dropped_beyond_their_number(folders):
+    from .gpu_engine import load_gpu_model
+    from trapetum_amd.engine.graphs import GraphedDecode
+    model, cfg = load_gpu_model(folders["A"], "bfloat16")
+    cache = model.new_cache(max_tokens=2048, max_slots=16)
+    graphed = GraphedDecode(model, cache, max_graphs=2)
+    slots = [cache.acquire() for _ in range(5)]
+    model.step(cache, slots, [1] * 5)
+    first = graphed.step(slots[:1], [3]).clone()
+    for n in (2, 3, 5, 1):                                       # rows 2, 4, 8, 1: the graph of one row was dropped and comes again
+        graphed.step(slots[:n], [3] * n)
+    assert len(graphed.graphs) == 2 and graphed.captures == 5
+    assert set(k[0] for k in graphed.graphs) == {8, 1}

@@ -9,6 +9,10 @@ size.  Entries with the same needs form a group with storage of its own:
                keeps a ring: position p lives in ring row p % rows_cap.
   state        [entries, slots, *shape], zeroed when a slot is taken.
 
+Beyond what sequences can take, every pool has one spare page and every state one
+spare slot (`ModelCache.spare_slot`): a row of a step that stands for no sequence
+(padding of a captured decode graph to its batch size) writes and reads there.
+
 The reference allocates cache_k / cache_v [max_seq, kv_heads * head_dim] per
 layer for its one sequence, K stored after RoPE (runtime/src/lib.rs:4475,
 :4488-4490), and models no window (:4455).
@@ -66,14 +70,16 @@ class CacheSite:
 
 
 class _KVGroup:
-    def __init__(self, spec, entries, n_pages, page_size, max_context, dtype, device, name):
+    def __init__(self, spec, entries, n_pages, max_slots, page_size, max_context, dtype, device, name):
         self.spec = spec
         self.entries = entries
         rows_cap = None
         if spec.window is not None and spec.window < max_context:
             rows_cap = -(-spec.window // page_size) * page_size
+            n_pages = min(n_pages, max_slots * (rows_cap // page_size))      # a ring never grows beyond its rows
         self.pages = GroupPages(n_pages, page_size, rows_cap, name)
-        shape = (len(entries), n_pages, spec.kv_heads, page_size, spec.head_dim)
+        self.spare_page = n_pages                                          # the pool's last page, never handed out
+        shape = (len(entries), n_pages + 1, spec.kv_heads, page_size, spec.head_dim)
         self.k_pool = torch.zeros(shape, dtype=dtype, device=device)
         self.v_pool = torch.zeros(shape, dtype=dtype, device=device)
         self.max_pages_per_seq = self.pages.max_pages(max_context)
@@ -84,7 +90,7 @@ class _StateGroup:
         self.spec = spec
         self.entries = entries
         dt = torch.float32 if spec.dtype == "float32" else dtype
-        self.tensor = torch.zeros((len(entries), max_slots) + tuple(spec.shape), dtype=dt, device=device)
+        self.tensor = torch.zeros((len(entries), max_slots + 1) + tuple(spec.shape), dtype=dt, device=device)
 
 
 class ModelCache:
@@ -102,6 +108,7 @@ class ModelCache:
         self.max_context = max_context
         self.max_tokens = max_tokens
         self.max_slots = max_slots
+        self.spare_slot = max_slots           # a slot no sequence takes: see the module's text
         n_pages = max(1, -(-max_tokens // page_size))
         self.kv_groups, self.state_groups = [], []
         self._site_of = {}
@@ -112,7 +119,7 @@ class ModelCache:
         for spec, entries in keyed.items():
             if isinstance(spec, KVSpec):
                 name = f"kv{len(self.kv_groups)}:" + ("all" if spec.window is None else f"window{spec.window}")
-                g = _KVGroup(spec, entries, n_pages, page_size, max_context, dtype, device, name)
+                g = _KVGroup(spec, entries, n_pages, max_slots, page_size, max_context, dtype, device, name)
                 gi = len(self.kv_groups)
                 self.kv_groups.append(g)
             elif isinstance(spec, StateSpec):
@@ -155,11 +162,15 @@ class ModelCache:
         return self.book.tokens_held(self.page_size)
 
     def page_table(self, group_index, slots, width=None):
-        """int32 [len(slots), width]: page ids of each slot in a group, -1 where it has none."""
+        """int32 [len(slots), width]: page ids of each slot in a group, -1 where it has none; the spare slot's row
+        names the spare page."""
         g = self.kv_groups[group_index]
         width = width or max(1, max(len(g.pages.lists.get(s, ())) for s in slots))
         t = np.full((len(slots), width), -1, dtype=np.int32)
         for i, s in enumerate(slots):
+            if s == self.spare_slot:
+                t[i, 0] = g.spare_page
+                continue
             p = g.pages.lists.get(s, ())
             t[i, :len(p)] = p
         return t

@@ -72,32 +72,38 @@ def step_arrays(cache, slots, counts, starts, want_rows, table_widths=None, key_
 
 class StaticStep:
     """Fixed device memory for the geometry of decode steps of one batch size, so that a captured HIP graph
-    finds every step's numbers at the same addresses.  Page tables have the cache's widest width."""
+    finds every step's numbers at the same addresses.  Page tables have the cache's widest width.  `extra` more
+    int32 follow the geometry for what else changes with the step (a sampler's uniform numbers, as bit patterns)."""
 
     RING = 8
 
-    def __init__(self, rt, cache, n_seq, length_bound):
+    def __init__(self, rt, cache, n_seq, extra=0):
         import torch
         self.rt = rt
         self.n_seq = n_seq
-        self.length_bound = length_bound        # the graph serves steps whose sequences are no longer than this
         self.table_widths = [g.max_pages_per_seq for g in cache.kv_groups]
-        size = 6 * n_seq + 1 + sum(n_seq * w for w in self.table_widths)
-        self.size = size
-        self.device_buffer = torch.zeros(size, dtype=torch.int32, device=rt.device)
-        self.pinned = [torch.zeros(size, dtype=torch.int32, pin_memory=True) for _ in range(self.RING)]
+        self.geometry = 6 * n_seq + 1 + sum(n_seq * w for w in self.table_widths)
+        self.size = self.geometry + extra
+        self.device_buffer = torch.zeros(self.size, dtype=torch.int32, device=rt.device)
+        self.pinned = [torch.zeros(self.size, dtype=torch.int32, pin_memory=True) for _ in range(self.RING)]
         self.events = [None] * self.RING
         self.turn = 0
 
-    def fill(self, flat):
+    def extra_view(self):
+        return self.device_buffer[self.geometry:]
+
+    def fill(self, flat, extra=None):
         """Queue the copy of this step's numbers into the fixed buffer (on the current stream)."""
         import torch
-        assert flat.size == self.size, (flat.size, self.size)
+        assert flat.size == self.geometry, (flat.size, self.geometry)
         i = self.turn
         self.turn = (i + 1) % self.RING
         if self.events[i] is not None:
             self.events[i].synchronize()
-        self.pinned[i].copy_(torch.from_numpy(flat))
+        self.pinned[i][:self.geometry].copy_(torch.from_numpy(flat))
+        if extra is not None:
+            assert extra.size == self.size - self.geometry
+            self.pinned[i][self.geometry:].copy_(torch.from_numpy(extra))
         self.device_buffer.copy_(self.pinned[i], non_blocking=True)
         ev = torch.cuda.Event()
         ev.record()
@@ -107,7 +113,9 @@ class StaticStep:
 class StepContext:
     """Everything parts need during a step.  Device tensors are int32."""
 
-    def __init__(self, rt, cache, slots, counts, starts, want_rows, static=None):
+    def __init__(self, rt, cache, slots, counts, starts, want_rows, static=None, length_bound=None):
+        """static: a StaticStep that the caller has filled with this step's numbers (a step captured in a graph reads
+        them there); length_bound: the longest sequence the captured launches must serve."""
         self.rt = rt
         self.ops = rt.ops
         self.dtype = rt.dtype
@@ -122,6 +130,7 @@ class StepContext:
         self.entry = None               # schedule entry now running
         self.cache_owner = None         # entry whose cache it uses
         self.static = static
+        self.length_bound = length_bound
         self._shared = set()            # entries whose step keys/values a later entry reads
         self._step_kv = {}
         n, m = self.n_seq, self.n_rows
@@ -131,7 +140,6 @@ class StepContext:
         flat, shapes = step_arrays(cache, self.slots, self.counts, self.starts, want_rows,
                                    static.table_widths if static is not None else None, self.key_geometry)
         if static is not None:
-            static.fill(flat)
             dev = static.device_buffer
         else:
             dev = rt.upload_i32(flat)
@@ -165,8 +173,8 @@ class StepContext:
         """Most keys any sequence of this step can see at this cache site (a host number, for launch geometry).
         With fixed step memory (a captured graph) it is the graph's bound on the lengths."""
         longest = max(s + c for s, c in zip(self.starts, self.counts))
-        if self.static is not None:
-            longest = max(longest, self.static.length_bound)
+        if self.length_bound is not None:
+            longest = max(longest, self.length_bound)
         return min(longest, site.rows_cap) if site.rows_cap else longest
 
     # keys and values of this step, for entries that read another entry's cache during a prefill

@@ -51,7 +51,7 @@ class Engine:
         limit = getattr(config, "max_position_embeddings", None)
         if max_context is None:
             max_context = min(max_tokens_in_cache, limit) if limit else max_tokens_in_cache
-        self.cache = model.new_cache(max_tokens_in_cache, max_context=max_context, page_size=page_size)
+        self.cache = model.new_cache(max_tokens_in_cache, max_context=max_context, max_slots=max_batch, page_size=page_size)
         self.graphed = None
         if use_graph and model.rt.device.type == "cuda":
             from .graphs import GraphedDecode
@@ -76,15 +76,17 @@ class Engine:
         return cls(model, config, stop_ids=(), **kw)
 
     def generate(self, prompts, max_tokens=256, temperature=0.0, top_p=0.95, top_k=256, repetition_penalty=1.0,
-                 seed=0, stop_ids=None, on_tokens=None, with_reasons=False):
-        """prompts: a list of token-id lists.  Returns the generated ids of each prompt."""
+                 seed=0, stop_ids=None, on_tokens=None, with_reasons=False, request_ids=None):
+        """prompts: a list of token-id lists.  Returns the generated ids of each prompt.  request_ids (integers, default
+        a prompt's place in the list) key the sampler's random numbers beside `seed`: a request keeps its tokens
+        whatever else is in the call if it keeps its id."""
         if prompts and isinstance(prompts[0], int):
             raise TypeError("prompts is a list of token-id lists (one list per request)")
         params = SamplingParams(temperature=temperature, top_p=top_p, top_k=top_k, repetition_penalty=repetition_penalty)
         stops = self.stop_ids if stop_ids is None else tuple(stop_ids)
         return _generate(self.model, self.cache, prompts, max_tokens=max_tokens, params=params, seed=seed,
                          stop_ids=stops, max_batch=self.max_batch, on_tokens=on_tokens, with_reasons=with_reasons,
-                         decode_step=self.graphed.step if self.graphed is not None else None)
+                         graphs=self.graphed, request_ids=request_ids)
 
 
 def load_model(folder, **kw):

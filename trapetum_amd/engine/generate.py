@@ -7,13 +7,22 @@ reference's (runtime/src/bin/gemma_run.rs:12-15, runtime/src/lib.rs:1574-1588): 
 it, choose the next; a stop token ends the sequence before it is emitted (runtime/src/bin/serve.rs:347-350),
 and the last emitted token is not run through the model.  The reference runs one sequence and truncates long
 prompts silently (serve.rs:323-326); here a prompt that cannot fit is an error.
+
+The chosen tokens stay on the device: a step reads the ids the step before chose, and the host reads them one
+step behind, after it has enqueued the next step, so the GPU does not wait for the host.  A sequence that turns
+out to have stopped has then run one step for nothing.  With captured graphs (`GraphedDecode`) the choice is
+part of the graph and a step is one copy of its numbers and one replay; without them the same loop runs eager
+steps.  There is one loop: `BatchRun` is what `generate` runs, and what the benchmark times.
 """
 import collections
 import dataclasses
 from typing import List
 
+import torch
+
 from ..cache.slots import CacheError
 from ..sampling.sampler import RequestSampling, Sampler, SamplingParams
+from .graphs import graph_rows
 
 
 @dataclasses.dataclass
@@ -50,21 +59,189 @@ def plan_batch(queue, prompts, max_tokens, max_batch, free_tokens, page_size, ma
     return taken
 
 
-def _index(like, rows):
-    import torch
-    return torch.tensor(rows, dtype=torch.long, device=like.device)
+class EagerRows:
+    """A batch's rows while it decodes, by eager steps: row r is the r-th sequence of the batch; `tokens[r]` is the
+    id it chose last."""
+
+    def __init__(self, model, cache, slots, sampler, requests):
+        self.model, self.cache, self.slots, self.sampler, self.requests = model, cache, slots, sampler, requests
+        self.tokens = None
+
+    def start(self, ids):
+        self.tokens = ids
+
+    def step(self, rows):
+        """Run the rows' last tokens through the model and choose their next ones."""
+        everyone = len(rows) == self.tokens.numel()
+        index = None if everyone else torch.tensor(rows, dtype=torch.long, device=self.tokens.device)
+        tok = self.tokens if everyone else self.tokens[index]
+        logits = self.model.step(self.cache, [self.slots[r] for r in rows], tok)
+        ids = self.sampler.choose_on_device(logits, [self.requests[r] for r in rows])
+        if everyone:
+            self.tokens = ids
+        else:
+            self.tokens = self.tokens.clone()
+            self.tokens[index] = ids
+
+    def fetch(self):
+        """Start the download of the rows' last ids; returns a function that waits for it and gives {row: id}."""
+        wait = self.model.rt.download_i32(self.tokens)
+        return lambda: dict(enumerate(wait()))
+
+
+class GraphRows:
+    """The same by graph replays.  A row keeps its place in the graph while its sequence lives; the places of
+    sequences that ended, and those beyond the batch, stand for no sequence (the cache's spare slot).  When half
+    of a graph's rows or fewer are left alive, the live ones move to the front of a graph of half the size."""
+
+    def __init__(self, graphs, model, cache, slots, sampler, requests):
+        self.graphs, self.model, self.cache, self.slots = graphs, model, cache, slots
+        self.requests = requests
+        self.choice = sampler.graph_choice()
+        self.nb = graph_rows(len(slots))
+        self.place = list(range(len(slots)))          # row -> place in the graph's rows
+
+    def start(self, ids):
+        self.graphs.rows(self.nb).tokens[:len(self.slots)].copy_(ids)
+
+    def step(self, rows):
+        cache = self.cache
+        nb = graph_rows(len(rows))
+        if nb < self.nb:                              # the live rows move into a smaller graph
+            old = self.graphs.rows(self.nb).tokens
+            index = torch.tensor([self.place[r] for r in rows], dtype=torch.long, device=old.device)
+            self.graphs.rows(nb).tokens[:len(rows)].copy_(old[index])
+            self.place = [None] * len(self.place)
+            for at, r in enumerate(rows):
+                self.place[r] = at
+            self.nb = nb
+        slots, starts = [cache.spare_slot] * self.nb, [0] * self.nb
+        uniforms = [0.5] * self.nb if self.choice[0] == "sample" else None
+        live = [self.slots[r] for r in rows]
+        cache.check_grow(live, [1] * len(live))
+        for r in rows:
+            at = self.place[r]
+            slots[at] = self.slots[r]
+            starts[at] = cache.grow(self.slots[r], 1)
+            if uniforms is not None:
+                uniforms[at] = self.requests[r].next_uniform()
+        self.graphs.run(self.nb, slots, starts, self.choice, uniforms)
+
+    def fetch(self):
+        wait = self.model.rt.download_i32(self.graphs.rows(self.nb).tokens)
+        place = list(self.place)
+        return lambda: (lambda ids: {r: ids[at] for r, at in enumerate(place) if at is not None})(wait())
+
+
+class BatchRun:
+    """One batch of requests from its prompts to its last token.
+
+    items: [(request index, prompt tokens, request id for the sampler)].  `prefill()` runs the prompts and chooses
+    every sequence's first token; each `advance()` enqueues one more decode step for the sequences that may go on
+    and then settles the tokens of the step before (stops, limits, slots given back); `done` when no sequence is left.
+    """
+
+    def __init__(self, model, cache, items, max_tokens, sampler, seed, stop, graphs=None):
+        self.model, self.cache, self.sampler = model, cache, sampler
+        self.items = items
+        self.max_tokens = max_tokens
+        self.stop = stop
+        self.requests = [RequestSampling(seed, rid, list(prompt)) for _, prompt, rid in items]
+        self.out = [[] for _ in items]
+        self.finished = {}                            # row -> Finished
+        self.slots = []
+        self.pending = None                           # (rows, wait): ids chosen on the device that the host has not read
+        self.rows = None
+        self.graphs = graphs if graphs is not None and sampler.graph_choice() is not None else None
+        self.steps = 0
+
+    @property
+    def done(self):
+        return self.pending is None
+
+    def prefill(self):
+        model, cache = self.model, self.cache
+        self.slots = [cache.acquire() for _ in self.items]
+        flat = [t for _, prompt, _ in self.items for t in prompt]
+        logits = model.step(cache, self.slots, flat, counts=[len(prompt) for _, prompt, _ in self.items])
+        ids = self.sampler.choose_on_device(logits, self.requests)
+        if self.graphs is not None:
+            self.rows = GraphRows(self.graphs, model, cache, self.slots, self.sampler, self.requests)
+        else:
+            self.rows = EagerRows(model, cache, self.slots, self.sampler, self.requests)
+        self.rows.start(ids)
+        self.pending = (list(range(len(self.items))), self.rows.fetch())
+
+    def _may_go_on(self, r, emitted):
+        """Whether row r, having emitted `emitted` tokens, runs its last token through the model for another one."""
+        return emitted < self.max_tokens and len(self.items[r][1]) + emitted <= self.cache.max_context
+
+    def _settle(self, rows, ids):
+        """The ids the rows chose: a stop token ends a row, any other is emitted; returns (emitted, rows that go on)."""
+        emitted, still = [], []
+        for r in rows:
+            tok, out = ids[r], self.out[r]
+            if tok in self.stop:
+                self.finished[r] = Finished(out, "stop")
+            else:
+                out.append(tok)
+                emitted.append((self.items[r][0], tok))
+                if len(out) >= self.max_tokens:
+                    self.finished[r] = Finished(out, "length")
+                elif len(self.items[r][1]) + len(out) > self.cache.max_context:
+                    self.finished[r] = Finished(out, "context")
+                else:
+                    still.append(r)
+            if r in self.finished:
+                self.cache.release(self.slots[r])
+                self.slots[r] = None
+        return emitted, still
+
+    def advance(self):
+        """Returns what the settled step emitted: [(request index, token)]."""
+        rows, wait = self.pending
+        if self.sampler.needs_the_last_token:
+            # the next choice looks at the tokens chosen so far: the host reads them before it goes on
+            ids = wait()
+            self.sampler.record([self.requests[r] for r in rows], [ids[r] for r in rows])
+            emitted, still = self._settle(rows, ids)
+            ahead = still
+            if ahead:
+                self.rows.step(ahead)
+        else:
+            # every row that its length allows to go on runs before the host knows what it chose last
+            ahead = [r for r in rows if self._may_go_on(r, len(self.out[r]) + 1)]
+            if ahead:
+                self.rows.step(ahead)
+            emitted, still = self._settle(rows, wait())
+            ahead = [r for r in ahead if r in still]
+        self.steps += 1
+        self.pending = (ahead, self.rows.fetch()) if ahead else None
+        return emitted
+
+    def close(self):
+        for i, s in enumerate(self.slots):
+            if s is not None:
+                self.cache.release(s)
+                self.slots[i] = None
+        self.pending = None
 
 
 def generate(model, cache, prompts, max_tokens=256, params=None, seed=0, stop_ids=(), max_batch=64,
-             on_tokens=None, with_reasons=False, decode_step=None):
+             on_tokens=None, with_reasons=False, graphs=None, request_ids=None):
     """Generate for every prompt (lists of token ids); returns the new tokens of each, in the prompts' order.
 
     on_tokens(step, [(request index, token), ...]) is called after every step with what it emitted.
-    decode_step(slots, tokens) -> logits replaces the model's step for the one-token steps (graph replay).
+    graphs: a GraphedDecode for the one-token steps.  request_ids: what the sampler's random numbers are keyed by
+    beside the seed (default: a request's place in `prompts`).
     """
     params = params or SamplingParams()
     sampler = Sampler(model.rt, params)
     stop = set(int(s) for s in stop_ids)
+    if request_ids is None:
+        request_ids = list(range(len(prompts)))
+    if len(request_ids) != len(prompts):
+        raise ValueError(f"{len(prompts)} prompts but {len(request_ids)} request ids")
     results = [None] * len(prompts)
     if max_tokens <= 0:
         for i in range(len(prompts)):
@@ -76,51 +253,17 @@ def generate(model, cache, prompts, max_tokens=256, params=None, seed=0, stop_id
         free = cache.max_tokens - cache.tokens_held()
         n = plan_batch(queue, prompts, max_tokens, max_batch, free, cache.page_size, cache.max_context)
         batch = [queue.popleft() for _ in range(n)]
-        slots = {i: cache.acquire() for i in batch}
-        state = {i: RequestSampling(seed, i, list(prompts[i])) for i in batch}
-        out = {i: [] for i in batch}
+        run = BatchRun(model, cache, [(i, prompts[i], int(request_ids[i])) for i in batch], max_tokens, sampler, seed,
+                       stop, graphs=graphs)
         try:
-            flat = [t for i in batch for t in prompts[i]]
-            logits = model.step(cache, [slots[i] for i in batch], flat, counts=[len(prompts[i]) for i in batch])
-            live = list(batch)
-            step = decode_step or (lambda sl, tk: model.step(cache, sl, tk))
-            while live:
-                requests = [state[i] for i in live]
-                ids = sampler.choose_on_device(logits, requests)
-                fetch = model.rt.download_i32(ids)
-                # The next step is enqueued before the host knows the tokens (they stay on the device), so the GPU
-                # does not wait for the host: every sequence that its length allows to go on takes part.  One that
-                # turns out to have stopped has run one step for nothing; its row is dropped below.
-                ahead = [i for i in live if len(out[i]) + 1 < max_tokens
-                         and len(prompts[i]) + len(out[i]) + 1 <= cache.max_context]
-                next_logits = None
-                if ahead:
-                    tokens = ids if len(ahead) == len(live) else ids[_index(ids, [live.index(i) for i in ahead])]
-                    next_logits = step([slots[i] for i in ahead], tokens)
-                chosen = fetch()
-                sampler.record(requests, chosen)
-                emitted, still = [], []
-                for i, tok in zip(live, chosen):
-                    if tok in stop:
-                        results[i] = Finished(out[i], "stop")
-                    else:
-                        out[i].append(tok)
-                        emitted.append((i, tok))
-                        if len(out[i]) >= max_tokens:
-                            results[i] = Finished(out[i], "length")
-                        elif len(prompts[i]) + len(out[i]) > cache.max_context:
-                            results[i] = Finished(out[i], "context")
-                        else:
-                            still.append(i)
-                    if results[i] is not None:
-                        cache.release(slots.pop(i))
+            run.prefill()
+            while not run.done:
+                emitted = run.advance()
                 if on_tokens is not None and emitted:
                     on_tokens(step_no, emitted)
                 step_no += 1
-                if still and len(still) != len(ahead):
-                    next_logits = next_logits[_index(next_logits, [ahead.index(i) for i in still])]
-                live, logits = still, next_logits
         finally:
-            for s in slots.values():
-                cache.release(s)
+            run.close()
+        for r, i in enumerate(batch):
+            results[i] = run.finished[r]
     return results if with_reasons else [r.tokens for r in results]

@@ -31,6 +31,8 @@ _CORE_SIGS = {
     "tp_repetition_penalty": [_P, _I, _I, _P, _I, _F, _P],
     "tp_sample": [_P, _I, _I, _F, _I, _F, _P, _P, _P, _P],
     "tp_sample_workspace_bytes": [_I, _I],
+    "tp_probe_stream": [_P, _L, _P, _I, _P],
+    "tp_probe_mfma": [_I, _I, _I, _P, _P, _P],
 }
 _ATTN_SIGS = {
     "tp_attn_prefill": [_P, _L, _P, _L, _P, _L, _I, _I, _I, _P, _I, _I, _P, _I, _I, _F, _F, _I, _P, _P, _P],
@@ -460,13 +462,18 @@ class HipOps:
         self._call(self.lib, "tp_repetition_penalty", logits.data_ptr(), logits.shape[0], logits.shape[1],
                    recent.data_ptr(), recent.shape[1], float(penalty), self._stream())
 
-    def sample(self, logits, temperature, top_k, top_p, uniforms):
+    def sample(self, logits, temperature, top_k, top_p, uniforms, out=None):
         self._dev(logits, uniforms)
         if logits.dtype != torch.float32 or logits.dim() != 2 or not logits.is_contiguous():
             raise KernelError("sample: logits must be contiguous float32 [rows, vocab]")
         if uniforms.dtype != torch.float32 or uniforms.numel() != logits.shape[0] or not uniforms.is_contiguous():
             raise KernelError("sample: one float32 uniform number per row")
-        out = torch.empty(logits.shape[0], dtype=torch.int32, device=self.device)
+        if out is None:
+            out = torch.empty(logits.shape[0], dtype=torch.int32, device=self.device)
+        else:
+            self._dev(out)
+            if out.dtype != torch.int32 or out.shape != (logits.shape[0],) or not out.is_contiguous():
+                raise KernelError("sample: the output must be contiguous int32 [rows]")
         # the candidate filter's workspace starts zeroed and every call leaves it zeroed again: kept between calls
         shape = tuple(logits.shape)
         if shape not in self._sample_ws:
@@ -477,3 +484,40 @@ class HipOps:
                    int(top_k), float(top_p), uniforms.data_ptr(), out.data_ptr(), ws.data_ptr() if ws is not None else None,
                    self._stream())
         return out
+
+    # ---- probes: what the GPU gives a kernel at best -----------------------------------------------------------
+    def _best_ms(self, launch, repeats):
+        launch()
+        torch.cuda.synchronize(self.device)
+        best = float("inf")
+        for _ in range(repeats):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            launch()
+            b.record()
+            b.synchronize()
+            best = min(best, a.elapsed_time(b))
+        return best
+
+    def measured_ceilings(self, stream_bytes=4 << 30, repeats=5):
+        """(GB/s of a streaming read of device memory, flop/s of a loop of bf16 matrix instructions), each the best
+        of a few runs of a probe kernel."""
+        cus = torch.cuda.get_device_properties(self.device).multi_processor_count
+        sink = torch.zeros(4, dtype=torch.float32, device=self.device)
+        buf = torch.empty(stream_bytes, dtype=torch.uint8, device=self.device).fill_(1)
+        ms = self._best_ms(lambda: self._call(self.lib, "tp_probe_stream", buf.data_ptr(), stream_bytes, sink.data_ptr(),
+                                              cus * 32, self._stream()), repeats)
+        gbs = stream_bytes / (ms * 1e-3) / 1e9
+        del buf
+        best, mhz = 0.0, 0.0
+        clocks = torch.zeros(2, dtype=torch.int64, device=self.device)
+        for kind in (0, 1):                            # the 16x16x32 and the 32x32x16 form of the instruction
+            iters, blocks = 20000, cus * 8
+            ms = self._best_ms(lambda: self._call(self.lib, "tp_probe_mfma", kind, iters, blocks, sink.data_ptr(),
+                                                  clocks.data_ptr(), self._stream()), repeats)
+            flops = blocks * 4 * iters * 131072.0 / (ms * 1e-3)
+            if flops > best:
+                c = clocks.tolist()
+                best, mhz = flops, (100.0 * c[0] / c[1] if c[1] else 0.0)
+        self.matrix_clock_mhz = mhz                    # the shader clock while the matrix loop ran
+        return gbs, best

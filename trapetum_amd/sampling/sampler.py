@@ -5,8 +5,10 @@ index winning ties (runtime/src/lib.rs:1376-1380); otherwise the top_k largest l
 (z - max) / T, the shortest prefix whose mass reaches top_p, and a draw r = u * kept mass walked down the
 sorted candidates.  A repetition penalty over the last 128 tokens, prompt included, comes first
 (serve.rs:285-294, :327-333).  The reference seeds one xorshift64 state from the clock (serve.rs:309-311);
-here every request owns a state derived from (seed, request index), so a request's draws do not depend on
-which other requests share its batch.  The logits never leave the device: only the chosen ids do.
+here every request owns a state derived from (seed, request id), the id being the caller's or else the
+request's place in the call, and draws one number per token of its own, so a request's draws do not depend on
+which other requests share its batch: the same request under the same id and seed gets the same tokens alone
+and in a batch.  The logits never leave the device: only the chosen ids do.
 """
 import collections
 import dataclasses
@@ -44,7 +46,7 @@ def xorshift64(state):
 
 
 def initial_state(seed, index):
-    """A non-zero 64-bit state from (seed, request index): splitmix64 over their mix."""
+    """A non-zero 64-bit state from (seed, request id): splitmix64 over their mix."""
     z = (seed * 0x9E3779B97F4A7C15 + (index + 1) * 0xBF58476D1CE4E5B9) & MASK64
     z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & MASK64
     z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & MASK64
@@ -55,8 +57,8 @@ def initial_state(seed, index):
 class RequestSampling:
     """What sampling remembers of one request."""
 
-    def __init__(self, seed, index, prompt):
-        self.state = initial_state(seed, index)
+    def __init__(self, seed, request_id, prompt):
+        self.state = initial_state(seed, request_id)
         self.recent = collections.deque(prompt[-RECENT_WINDOW:], maxlen=RECENT_WINDOW)
 
     def next_uniform(self):
@@ -72,6 +74,20 @@ class Sampler:
         params.validate()
         self.rt = rt
         self.params = params
+
+    @property
+    def needs_the_last_token(self):
+        """Whether a choice depends on the tokens chosen before it (then the host must know them first)."""
+        return self.params.repetition_penalty > 1.0
+
+    def graph_choice(self):
+        """The choice as a captured decode graph can make it by itself (see GraphedDecode.run), or None."""
+        p = self.params
+        if self.needs_the_last_token:
+            return None
+        if p.temperature <= 0:
+            return ("greedy",)
+        return ("sample", float(p.temperature), int(p.top_k), float(p.top_p))
 
     def choose(self, logits, requests):
         """logits fp32 [n, vocab] on the device (changed in place by a penalty); one RequestSampling per row.

@@ -62,13 +62,17 @@ class RandomWeights:
         return (t * sigma).to(self.store_dtype)
 
 
-def write_model_folder(config, folder, seed, sigma=0.02, sigma_norm=0.1):
-    """Write config.json and model.safetensors of a randomly initialised model of `config`."""
+def write_model_folder(config, folder, seed, sigma=0.02, sigma_norm=0.1, store_dtype="bfloat16"):
+    """Write config.json and model.safetensors of a randomly initialised model of `config`.  store_dtype
+    "bfloat16" rounds the drawn values to bfloat16; "float32" stores them as drawn (and the engine keeps them so)."""
     from ..engine.model import Model
     from ..registry import architecture
+    widths = {"bfloat16": torch.bfloat16, "float32": torch.float32}
+    if store_dtype not in widths:
+        raise ValueError(f"store_dtype '{store_dtype}' must be bfloat16 or float32")
     arch = architecture(config.architecture)
     layout = Model(arch.build_spec(config), rt=None).tensor_layout()
-    source = RandomWeights(layout, seed, sigma, sigma_norm)
+    source = RandomWeights(layout, seed, sigma, sigma_norm, store_dtype=widths[store_dtype])
     os.makedirs(folder, exist_ok=True)
     with open(os.path.join(folder, "config.json"), "w") as f:
         json.dump(config.to_dict(), f, indent=1)
