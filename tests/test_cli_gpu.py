@@ -1,0 +1,76 @@
+"""The command line as a user runs it: `python -m trapetum_amd random`, then `run` and `generate` on the folder it
+wrote, and `run --random`; the ids must be the plain implementation's (the reference's entry point is such a
+binary: runtime/src/bin/gemma_run.rs:1-19)."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+from .plain import gemma2_plain as plain
+from .tiny import TINY_A, TINY_A_INIT, random_tokens
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def cli(*args):
+    p = subprocess.run([sys.executable, "-m", "trapetum_amd"] + [str(a) for a in args], cwd=ROOT, capture_output=True,
+                       text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    return p.stdout
+
+
+def test_random_run_generate(tmp_path):
+    config = tmp_path / "config.json"
+    config.write_text(json.dumps(dict(TINY_A, architectures=["Gemma2ForCausalLM"])))
+    folder = tmp_path / "model"
+    init = ["--seed", TINY_A_INIT["seed"], "--sigma", TINY_A_INIT["sigma"], "--sigma-norm", TINY_A_INIT["sigma_norm"]]
+    assert "wrote" in cli("random", "--config", config, "--out", folder, *init)
+    pcfg, pw = plain.read_folder(str(folder))
+    prompts = [random_tokens(n, pcfg["vocab_size"], 90 + n) for n in (5, 11, 17)]
+    want = [plain.greedy_generate(pcfg, pw, p, 8) for p in prompts]
+    ids_file = tmp_path / "prompt.bin"
+    np.asarray(prompts[1], dtype="<i4").tofile(ids_file)
+    out = cli("run", folder, ids_file, "--max-tokens", 8, "--dtype", "float32", "--no-stop")
+    assert out.strip() == f"continuation ids: {want[1]}"
+    out = cli("run", folder, "--prompt-ids", ",".join(map(str, prompts[0])), "--max-tokens", 8, "--dtype", "float32", "--no-stop")
+    assert out.strip() == f"continuation ids: {want[0]}"
+    lines = tmp_path / "prompts.txt"
+    lines.write_text("".join(" ".join(map(str, p)) + "\n" for p in prompts))
+    out = cli("generate", folder, "--prompts-file", lines, "--max-tokens", 8, "--dtype", "float32", "--no-stop")
+    assert [[int(t) for t in l.split()] for l in out.strip().splitlines()] == want
+    # the same model without a folder: random weights of the configuration, by the same seed
+    out = cli("run", "--random", config, "--weights-seed", TINY_A_INIT["seed"], "--sigma", TINY_A_INIT["sigma"],
+              "--sigma-norm", TINY_A_INIT["sigma_norm"], "--prompt-ids", ",".join(map(str, prompts[2])), "--max-tokens", 8,
+              "--dtype", "float32", "--no-stop")
+    assert out.strip() == f"continuation ids: {want[2]}"
+    # a stop token ends the continuation before it
+    out = cli("run", folder, "--prompt-ids", ",".join(map(str, prompts[1])), "--max-tokens", 8, "--dtype", "float32",
+              "--stop-id", want[1][3])
+    assert out.strip() == f"continuation ids: {want[1][:want[1].index(want[1][3])]}"
+
+
+def test_float32_weights_are_kept_as_drawn(tmp_path):
+    """`random --store-dtype float32` stores the drawn values unrounded, and the float32 engine keeps them so: its
+    logits follow a plain run on the unrounded values, not one on their bfloat16 roundings."""
+    import torch
+
+    from .tiny import rel_l2
+    config = tmp_path / "config.json"
+    config.write_text(json.dumps(dict(TINY_A, architectures=["Gemma2ForCausalLM"])))
+    folder = tmp_path / "model32"
+    cli("random", "--config", config, "--out", folder, "--seed", 4, "--sigma", 0.05, "--sigma-norm", 0.2, "--store-dtype", "float32")
+    pcfg, pw = plain.read_folder(str(folder))
+    assert any((t.float().to(torch.bfloat16).double() != t).any() for t in pw.values())     # not bfloat16 values
+    from .gpu_engine import load_gpu_model
+    model, cfg = load_gpu_model(str(folder), "float32")
+    toks = random_tokens(30, cfg.vocab_size, 8)
+    cache = model.new_cache(max_tokens=64)
+    s = cache.acquire()
+    got = model.step(cache, [s], toks, counts=[30], want=list(range(30)))
+    assert rel_l2(got, plain.forward(pcfg, pw, toks)) < 1e-5
+    rounded = {k: v.float().to(torch.bfloat16).double() for k, v in pw.items()}
+    assert rel_l2(got, plain.forward(pcfg, rounded, toks)) > 1e-4

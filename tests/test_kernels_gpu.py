@@ -86,6 +86,28 @@ def test_deferred_product_into_add_rms_norm(ops, m, n, k):
     assert rel_l2(stream, ref_stream) < 1e-5 and rel_l2(got, ref) < 6e-3
 
 
+def test_rows_wider_than_the_fused_kernel_takes_are_added_first(ops):
+    """A product in K slices whose rows are wider than `add_rms_norm` keeps in registers (8192): the slices are added by
+    a kernel of their own, in slice order, and the result is what the fused path gives for narrower rows."""
+    m, d = 5, 8192 + 8
+    slices = randn(3, m, d, seed=70)
+    stream = randn(m, d, seed=71)
+    gp, gn = randn(d, seed=72).abs() + 0.5, randn(d, seed=73).abs() + 0.5
+    ref_stream = stream.cpu().clone()
+    ref = ref_ops.add_rms_norm(ref_stream, slices.cpu().sum(0), gp.cpu(), 1e-5, gn.cpu(), 1e-6, torch.bfloat16)
+    from trapetum_amd.kernels.ops import SplitRows
+    got = ops.add_rms_norm(stream, SplitRows(slices), gp, 1e-5, gn, 1e-6, torch.bfloat16)
+    assert rel_l2(stream, ref_stream) < 3e-3 and rel_l2(got, ref) < 6e-3
+    summed = ops.rows(SplitRows(slices), torch.float32)
+    assert torch.equal(summed.cpu(), (slices[0] + slices[1] + slices[2]).cpu())
+    # a product may leave its slices to the consumer only without an epilogue
+    x, w = randn(8, 64, dtype=torch.bfloat16, seed=74), randn(128, 64, dtype=torch.bfloat16, seed=75)
+    y = torch.empty(8, 128, dtype=torch.float32, device=DEV)
+    ws = torch.empty(1 << 20, dtype=torch.uint8, device=DEV)
+    rc = ops.lib.tp_linear(x.data_ptr(), w.data_ptr(), y.data_ptr(), 1, 0, 8, 128, 64, 1, 30.0, 0, ws.data_ptr(), 1 << 20, 1, 0, None)
+    assert rc != 0 and b"epilogue" in ops.lib.tp_last_error()
+
+
 def test_gather_rows(ops):
     x = randn(9, 88)
     rows = torch.tensor([8, 0, 3, 3], dtype=torch.int32, device=DEV)

@@ -282,6 +282,7 @@ static int add_rms_norm_launch(float* stream, const void* rows, int n_slices, lo
     const bool aligned = D % 4 == 0 && (uintptr_t)rows % 16 == 0 && (uintptr_t)stream % 16 == 0 && slice_stride % 4 == 0 &&
                          (!gp || (uintptr_t)gp % 16 == 0) && (!gn || (uintptr_t)gn % 16 == 0) && (!out || (uintptr_t)out % 16 == 0);
     const bool few = aligned && M <= 128, vec = aligned && M > 128;
+    // (HipOps.add_rms_norm adds the slices itself, with sum_slices, before it comes here with a wider row)
 #define TP_ADD_NORM_VEC(CPT, NTH) add_rms_norm_vec_k<TR, T, CPT, NTH><<<M, NTH, 0, s>>>(stream, (const TR*)rows, n_slices, slice_stride, gp, ep, gn, en, (T*)out, D)
     if (few && D > 256 * 4 && D <= 640 * 4) TP_ADD_NORM_VEC(1, 640);
     else if (few && D > 640 * 4 && D <= 1024 * 4) TP_ADD_NORM_VEC(1, 1024);
@@ -315,6 +316,25 @@ extern "C" int tp_add_rms_norm(float* stream, const void* rows, int rows_dtype, 
     else return tp_fail("add_rms_norm: unsupported dtypes rows %d -> out %d", rows_dtype, out_dtype);
     if (rc) return rc;
     return tp_check_launch("add_rms_norm");
+}
+
+// ---- the K slices of a product added in slice order (for a consumer that does not add them itself) --------------
+template <typename T>
+__global__ void sum_slices_k(const float* __restrict__ slices, int n_slices, long slice_stride, T* __restrict__ out, long count) {
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (long)gridDim.x * blockDim.x) {
+        float t = 0.f;
+        for (int s = 0; s < n_slices; s++) t += slices[(size_t)s * slice_stride + i];
+        st_f32(out + i, t);
+    }
+}
+
+extern "C" int tp_sum_slices(const float* slices, int n_slices, long slice_stride, void* out, int out_dtype, long count, void* stream) {
+    TP_REQUIRE(slices && out && n_slices >= 1 && count > 0 && slice_stride >= count, "sum_slices: %d slices of %ld elements, %ld apart", n_slices, count, slice_stride);
+    const int blocks = (int)((count + 255) / 256 < 4096 ? (count + 255) / 256 : 4096);
+    if (out_dtype == TP_BF16) sum_slices_k<bf16_t><<<blocks, 256, 0, (hipStream_t)stream>>>(slices, n_slices, slice_stride, (bf16_t*)out, count);
+    else if (out_dtype == TP_F32) sum_slices_k<float><<<blocks, 256, 0, (hipStream_t)stream>>>(slices, n_slices, slice_stride, (float*)out, count);
+    else return tp_fail("sum_slices: unknown dtype %d", out_dtype);
+    return tp_check_launch("sum_slices");
 }
 
 // ---- gather rows of the fp32 stream -------------------------------------------------------------------

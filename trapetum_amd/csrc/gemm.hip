@@ -96,6 +96,7 @@ static int check_args(const GemmArgs& a) {
     TP_REQUIRE(a.out_dtype == TP_F32 || a.out_dtype == TP_BF16, "linear: unknown output dtype %d", a.out_dtype);
     TP_REQUIRE(!(a.in_dtype == TP_F32 && a.out_dtype == TP_BF16), "linear: float32 rows give float32 output");
     TP_REQUIRE(a.epilogue != TP_EPI_SOFTCAP || a.cap > 0.f, "linear: a soft cap must be positive");
+    TP_REQUIRE(!a.defer || a.epilogue == TP_EPI_NONE, "linear: K slices can be left to the consumer only without an epilogue (found %d)", a.epilogue);
     if (a.epilogue == TP_EPI_GATED) {
         const int padded = 2 * ((a.units + 15) / 16) * 16;
         TP_REQUIRE(a.units > 0 && a.N == padded, "gated product: %d units need a packed matrix of %d rows, found %d", a.units, padded, a.N);

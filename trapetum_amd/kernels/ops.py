@@ -18,6 +18,7 @@ _CORE_SIGS = {
     "tp_rms_norm": [_P, _I, _P, _F, _P, _I, _I, _I, _P],
     "tp_add_rms_norm": [_P, _P, _I, _I, _L, _P, _F, _P, _F, _P, _I, _I, _I, _P],
     "tp_gather_rows": [_P, _P, _P, _I, _I, _I, _P],
+    "tp_sum_slices": [_P, _I, _L, _P, _I, _L, _P],
     "tp_rope_kv_write": [_P, _L, _P, _L, _P, _L, _I, _I, _I, _I, _I, _P, _I, _P, _P, _P, _P, _I, _P, _P, _I, _I,
                          _P, _P, _L, _P, _P],
     "tp_gather_kv_prefix": [_P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P, _P, _P, _I, _P, _P, _L, _P],
@@ -164,6 +165,8 @@ class HipOps:
         """stream += post-norm(rows) (or rows); returns next-norm(stream) or None.  rows: a tensor or SplitRows."""
         m, d = stream.shape
         n_slices, stride = 1, 0
+        if isinstance(rows, SplitRows) and d > self.MAX_SLICED_WIDTH:
+            rows = self.rows(rows, out_dtype)            # the fused kernel keeps a row in registers: wider rows are added first
         if isinstance(rows, SplitRows):
             n_slices, stride = rows.slices.shape[0], rows.slices.stride(0)
             rows = rows.slices[0]
@@ -182,11 +185,20 @@ class HipOps:
                    out.data_ptr() if out is not None else None, _code(out_dtype), m, d, self._stream())
         return out
 
+    MAX_SLICED_WIDTH = 8192        # widest row `add_rms_norm` takes in K slices
+
     def rows(self, rows, dtype):
-        """A tensor of `dtype` from what `linear` returned."""
-        if isinstance(rows, SplitRows):
-            return rows.slices.sum(dim=0).to(dtype)
-        return rows
+        """A tensor of `dtype` from what `linear` returned: K slices are added in slice order."""
+        if not isinstance(rows, SplitRows):
+            return rows
+        sl = rows.slices
+        self._dev(sl)
+        if sl.dtype != torch.float32 or sl.dim() != 3 or not sl.is_contiguous():
+            raise KernelError("rows: K slices must be contiguous float32 [slices, rows, columns]")
+        out = torch.empty(sl.shape[1:], dtype=dtype, device=self.device)
+        self._call(self.lib, "tp_sum_slices", sl.data_ptr(), sl.shape[0], sl.stride(0), out.data_ptr(), _code(dtype),
+                   out.numel(), self._stream())
+        return out
 
     def gather_rows(self, x, rows):
         self._dev(x, rows)
@@ -307,8 +319,7 @@ class HipOps:
 
     # ---- attention -------------------------------------------------------------------------------------
     def _fast_attention(self, dtype, H, KV, hd):
-        return (not self.force_plain_attention and dtype == torch.bfloat16 and hd % 16 == 0 and hd <= 256
-                and H // KV <= 16 and _build.ATTN_SOURCE in _build.os.listdir(_build.CSRC))
+        return not self.force_plain_attention and dtype == torch.bfloat16 and hd % 16 == 0 and hd <= 256 and H // KV <= 16
 
     def attention_prefill(self, q, k, v, H, KV, hd, cu_rows, max_count, scale, softcap, window, out_dtype,
                           row_seq=None, row_pos=None, keys=None):
