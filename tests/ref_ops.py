@@ -54,11 +54,11 @@ def _gelu_tanh(g):
 
 
 def gated_linear(x, w_packed, inter, activation, out_dtype):
-    assert activation == "gelu_tanh"
+    act = {"gelu_tanh": _gelu_tanh, "silu": lambda g: g * torch.sigmoid(g)}[activation]
     y = x.float() @ w_packed.float().T                     # [M, 2 * ip]
     y = y.reshape(x.shape[0], -1, 2, GROUP)
     g, u = y[:, :, 0, :].reshape(x.shape[0], -1), y[:, :, 1, :].reshape(x.shape[0], -1)
-    return (_gelu_tanh(g) * u)[:, :inter].to(out_dtype).contiguous()
+    return (act(g) * u)[:, :inter].to(out_dtype).contiguous()
 
 
 def _rotate(x, pos, inv_freq, rotary_dim):

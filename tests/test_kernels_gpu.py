@@ -104,7 +104,7 @@ def test_rows_wider_than_the_fused_kernel_takes_are_added_first(ops):
     x, w = randn(8, 64, dtype=torch.bfloat16, seed=74), randn(128, 64, dtype=torch.bfloat16, seed=75)
     y = torch.empty(8, 128, dtype=torch.float32, device=DEV)
     ws = torch.empty(1 << 20, dtype=torch.uint8, device=DEV)
-    rc = ops.lib.tp_linear(x.data_ptr(), w.data_ptr(), y.data_ptr(), 1, 0, 8, 128, 64, 1, 30.0, 0, ws.data_ptr(), 1 << 20, 1, 0, None)
+    rc = ops.lib.tp_linear(x.data_ptr(), w.data_ptr(), y.data_ptr(), 1, 0, 8, 128, 64, 1, 30.0, 0, 0, ws.data_ptr(), 1 << 20, 1, 0, None)
     assert rc != 0 and b"epilogue" in ops.lib.tp_last_error()
 
 
@@ -183,11 +183,15 @@ def test_gated_linear(ops, algo, dt, m, inter, k):
     ops.force_linear = algo
     try:
         got = ops.gated_linear(x, packed, inter, "gelu_tanh", DT[dt])
+        silu = ops.gated_linear(x, packed, inter, "silu", DT[dt])
+        with pytest.raises(Exception, match="no kernel"):
+            ops.gated_linear(x, packed, inter, "relu", DT[dt])
     finally:
         ops.force_linear = 0
     g, u = x.cpu().double() @ wg.cpu().double().T, x.cpu().double() @ wu.cpu().double().T
     ref = torch.nn.functional.gelu(g, approximate="tanh") * u
     assert rel_l2(got, ref) < (5e-6 if dt == "f32" else 4e-3)
+    assert rel_l2(silu, torch.nn.functional.silu(g) * u) < (5e-6 if dt == "f32" else 4e-3)      # the other activation offered
 
 
 @pytest.mark.parametrize("algo,m", [(2, 8), (3, 8), (3, 200)])

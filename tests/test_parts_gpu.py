@@ -206,7 +206,7 @@ def test_the_gate_is_what_the_activation_is_applied_to(rt, m):
 
 def test_sandwich_block(rt):
     tol = 5e-6 if rt.dtype == torch.float32 else 1.5e-2
-    make_norm = lambda: build_part("norm", ("rms_norm", {"size": 88, "eps": 1e-5, "weight_offset": 1.0}))
+    make_norm = lambda site=None: build_part("norm", ("rms_norm", {"size": 88, "eps": 1e-5, "weight_offset": 1.0}))
     block = part_class("block", "sandwich")(build_part("mixer", ("attention", dict(ATT, window=None))),
                                             build_part("feed_forward", ("gated_mlp", {"hidden_size": 88, "intermediate_size": 200, "activation": "gelu_tanh"})),
                                             make_norm)

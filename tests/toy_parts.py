@@ -1,6 +1,6 @@
 """Toy parts defined by the tests, registered from outside the framework: a mixer with a state of fixed size
-per sequence, another position table, a feed-forward with a router over experts, and an architecture that mixes
-them with the built-in parts.  They are no model of anyone's; they show that the framework's files need no change
+per sequence, another position table, a feed-forward with a router over experts, a norm of another kind, and an
+architecture that mixes them with the built-in parts (one layer has two kinds of norm and a SiLU-gated feed-forward).  They are no model of anyone's; they show that the framework's files need no change
 for a new part."""
 import dataclasses
 import math
@@ -10,7 +10,7 @@ import torch
 from trapetum_amd.cache import StateSpec
 from trapetum_amd.config.base import ModelConfig, key
 from trapetum_amd.models.spec import LayerSpec, ModelSpec, ScheduleEntry, TensorSpec
-from trapetum_amd.parts import FeedForward, Mixer, Position
+from trapetum_amd.parts import FeedForward, Mixer, Norm, Position
 from trapetum_amd.registry import build_part, register_architecture, register_part
 
 
@@ -76,6 +76,27 @@ class SoftRoutedMLP(FeedForward):
         return out.to(ctx.dtype)
 
 
+class CenteredNorm(Norm):
+    """(x - mean) / sqrt(var + eps) * w + b: a norm with a shift, which no RMS kernel fuses (it exposes no `gain`), so
+    a block calls it through `forward` around a plain add."""
+
+    def __init__(self, size, eps):
+        self.size, self.eps = size, float(eps)
+
+    def tensor_specs(self):
+        return {"weight": TensorSpec((self.size,), init="norm"), "bias": TensorSpec((self.size,), init="norm")}
+
+    def bind(self, tensors, rt):
+        self.rt = rt
+        self.w, self.b = tensors["weight"].float(), tensors["bias"].float()
+
+    def forward(self, ctx, x, out_dtype=None):
+        x = x.float()
+        c = x - x.mean(-1, keepdim=True)
+        y = c * torch.rsqrt((c * c).mean(-1, keepdim=True) + self.eps) * (1.0 + self.w) + self.b
+        return y.to(out_dtype or ctx.dtype)
+
+
 class SquaredPosition(Position):
     """Rotary frequencies d -> 1 / (1 + d)^2 over part of the head: another table through the same interface."""
 
@@ -113,11 +134,13 @@ def toy_spec(c):
             mixer = ("attention", {"hidden_size": c.width, "num_heads": c.heads, "num_kv_heads": c.heads,
                                    "head_dim": c.head_size, "query_scale": 1.0 / math.sqrt(c.head_size),
                                    "position": ("toy_squared", {"rotary_dim": c.rotary})})
-        if l % 2 == 0:
-            ff = ("gated_mlp", {"hidden_size": c.width, "intermediate_size": c.ff_width, "activation": "gelu_tanh"})
+        norms = None
+        if l % 2 == 0:      # a SiLU gate, and a second kind of norm in front of it
+            ff = ("gated_mlp", {"hidden_size": c.width, "intermediate_size": c.ff_width, "activation": "silu"})
+            norms = {"pre_ff_norm": ("toy_centered_norm", {"size": c.width, "eps": c.eps})}
         else:
             ff = ("toy_soft_routed", {"hidden_size": c.width, "intermediate_size": c.ff_width, "n_experts": c.experts})
-        layers.append(LayerSpec(block=("pre_norm", {}), mixer=mixer, feed_forward=ff, norm=norm,
+        layers.append(LayerSpec(block=("pre_norm", {}), mixer=mixer, feed_forward=ff, norm=norm, norms=norms,
                                 prefixes={"pre_mixer_norm": p + "n1.", "mixer": p + "mix.", "pre_ff_norm": p + "n2.",
                                           "feed_forward": p + "ff."}))
     # the order of running is data: layer 0 runs twice (its second run keeps a state of its own), and the
@@ -133,6 +156,7 @@ def toy_spec(c):
 def register():
     register_part("mixer", "toy_ema", EmaMixer)
     register_part("position", "toy_squared", SquaredPosition)
+    register_part("norm", "toy_centered_norm", CenteredNorm)
     register_part("feed_forward", "toy_soft_routed", SoftRoutedMLP)
     register_architecture(ToyConfig.architecture, ToyConfig, toy_spec)
 
@@ -190,12 +214,16 @@ def toy_reference(cfg, W, tokens):
             a, kv = attn(n, p, kv1 if reuse else None)
             kv1 = kv1 or kv
             x = x + a
-        n = norm(x, W[p + "n2.weight"])
-
-        def mlp(t, q):
-            return (gelu(t @ W[q + "gate_proj.weight"].T) * (t @ W[q + "up_proj.weight"].T)) @ W[q + "down_proj.weight"].T
         if l == 0:
-            x = x + mlp(n, p + "ff.")
+            c = x - x.mean(-1, keepdim=True)
+            n = c * torch.rsqrt((c * c).mean(-1, keepdim=True) + cfg["eps"]) * (1 + W[p + "n2.weight"]) + W[p + "n2.bias"]
+        else:
+            n = norm(x, W[p + "n2.weight"])
+
+        def mlp(t, q, act=gelu):
+            return (act(t @ W[q + "gate_proj.weight"].T) * (t @ W[q + "up_proj.weight"].T)) @ W[q + "down_proj.weight"].T
+        if l == 0:
+            x = x + mlp(n, p + "ff.", lambda g: g * torch.sigmoid(g))
         else:
             mix = torch.softmax(n @ W[p + "ff.router.weight"].T, -1)
             x = x + sum(mix[:, e:e + 1] * mlp(n, p + f"ff.experts.{e}.") for e in range(cfg["experts"]))

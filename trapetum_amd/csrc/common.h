@@ -71,3 +71,22 @@ __device__ __forceinline__ float gelu_tanh_fast(float g) {
     constexpr float C1 = -2.f * 0.7978845608f * 1.4426950408889634f, C3 = C1 * 0.044715f;
     return g * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(g * __builtin_fmaf(C3, g * g, C1)));
 }
+
+// ---- gate activations of a gated product -----------------------------------------------------------------------
+// The activations offered are of one form, act(g) = g / (1 + 2^(g (c1 + c3 g^2))): gelu-tanh (above) with
+// c1 = -2 * 0.7978845608 * log2(e), c3 = c1 * 0.044715, and SiLU, g / (1 + e^-g), with c1 = -log2(e), c3 = 0.  The
+// bf16 products' epilogues take the two constants (`epi.x`, `epi.y`) and have no branch on the activation's kind.
+enum { TP_ACT_GELU_TANH = 0, TP_ACT_SILU = 1 };
+static inline bool tp_gate_constants(int act, float* c1, float* c3) {
+    constexpr float LOG2E = 1.4426950408889634f;
+    if (act == TP_ACT_GELU_TANH) { *c1 = -2.f * 0.7978845608f * LOG2E; *c3 = *c1 * 0.044715f; return true; }
+    if (act == TP_ACT_SILU) { *c1 = -LOG2E; *c3 = 0.f; return true; }
+    return false;
+}
+__device__ __forceinline__ float gate_act_fast(float g, float2 epi) {
+    return g * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(g * __builtin_fmaf(epi.y, g * g, epi.x)));
+}
+// the same in full float32 arithmetic, for the float32 path
+__device__ __forceinline__ float gate_act_exact(float g, int act) {
+    return act == TP_ACT_SILU ? g / (1.f + expf(-g)) : gelu_tanh_f(g);
+}

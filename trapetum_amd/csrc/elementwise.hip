@@ -510,23 +510,25 @@ extern "C" int tp_gather_kv_prefix(const void* k_pool, const void* v_pool, int d
 }
 
 // ---- gated activation on a packed gate/up product: y [M, 2*Ip] fp32 with 16 gate columns, then the 16 up
-// columns of the same units, alternating.  out[m, i] = gelu_tanh(g) * u (runtime/cuda/codebook_gemv.cu:531-537).
+// columns of the same units, alternating.  out[m, i] = act(g) * u, act being gelu-tanh (runtime/cuda/codebook_gemv.cu:
+// 531-537) or SiLU (the reference's other feed-forward: runtime/cuda/codebook_gemv.cu:205-209), in float32 arithmetic.
 template <typename T>
-__global__ void gated_act_k(const float* __restrict__ y, T* __restrict__ out, int I, int Ip2) {
+__global__ void gated_act_k(const float* __restrict__ y, T* __restrict__ out, int I, int Ip2, int act) {
     const float* yr = y + (size_t)blockIdx.x * Ip2;
     T* orow = out + (size_t)blockIdx.x * I;
     for (int i = threadIdx.x; i < I; i += blockDim.x) {
         const int base = (i >> 4) * 32 + (i & 15);
-        st_f32(orow + i, gelu_tanh_f(yr[base]) * yr[base + 16]);
+        st_f32(orow + i, gate_act_exact(yr[base], act) * yr[base + 16]);
     }
 }
 
-extern "C" int tp_gated_act(const float* y, void* out, int dtype, int M, int I, void* stream) {
+extern "C" int tp_gated_act(const float* y, void* out, int dtype, int M, int I, int act, void* stream) {
     TP_REQUIRE(M > 0 && I > 0, "gated_act: empty shape M=%d I=%d", M, I);
+    TP_REQUIRE(act == TP_ACT_GELU_TANH || act == TP_ACT_SILU, "gated_act: unknown activation %d", act);
     const int Ip2 = 2 * ((I + 15) / 16) * 16;
     hipStream_t s = (hipStream_t)stream;
-    if (dtype == TP_BF16) gated_act_k<bf16_t><<<M, 256, 0, s>>>(y, (bf16_t*)out, I, Ip2);
-    else if (dtype == TP_F32) gated_act_k<float><<<M, 256, 0, s>>>(y, (float*)out, I, Ip2);
+    if (dtype == TP_BF16) gated_act_k<bf16_t><<<M, 256, 0, s>>>(y, (bf16_t*)out, I, Ip2, act);
+    else if (dtype == TP_F32) gated_act_k<float><<<M, 256, 0, s>>>(y, (float*)out, I, Ip2, act);
     else return tp_fail("gated_act: unknown dtype %d", dtype);
     return tp_check_launch("gated_act");
 }

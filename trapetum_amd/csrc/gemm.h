@@ -11,11 +11,19 @@ struct GemmArgs {
     int M, N, K;            // N counts rows of W (for a gated product: 2 * padded units)
     int epilogue; float cap;
     int units;              // gated: columns of the output (the feed-forward width)
+    int act;                // gated: the gate's activation (TP_ACT_*)
     void* workspace; size_t workspace_bytes;
     int defer;              // split products: leave the K slices in the workspace [slices, M, N] for the consumer to add
     int algo;               // the caller's choice of kernel (0: none; see tp_linear)
     hipStream_t stream;
 };
+
+// the constants a kernel's epilogue takes: the cap, or the gate activation's two
+static inline float2 epi_constants(const GemmArgs& a) {
+    float2 e = make_float2(a.cap, 0.f);
+    if (a.epilogue == TP_EPI_GATED) tp_gate_constants(a.act, &e.x, &e.y);
+    return e;
+}
 
 // plain tiled kernel, any dtype and shape; one fixed summation order per output element
 int gemm_simple_launch(const GemmArgs& a);

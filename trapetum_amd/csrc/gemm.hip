@@ -55,7 +55,7 @@ gemm_simple_k(const TI* __restrict__ X, const TI* __restrict__ W, TO* __restrict
     }
 }
 
-extern "C" int tp_gated_act(const float* y, void* out, int dtype, int M, int I, void* stream);
+extern "C" int tp_gated_act(const float* y, void* out, int dtype, int M, int I, int act, void* stream);
 
 template <typename TI>
 static int simple_typed(const GemmArgs& a, void* y, int out_dtype, float cap) {
@@ -86,7 +86,7 @@ int gemm_simple_launch(const GemmArgs& a) {
     const float cap = a.epilogue == TP_EPI_SOFTCAP ? a.cap : 0.f;
     int rc = a.in_dtype == TP_BF16 ? simple_typed<bf16_t>(a, y, out_dtype, cap) : simple_typed<float>(a, y, out_dtype, cap);
     if (rc) return rc;
-    if (a.epilogue == TP_EPI_GATED) return tp_gated_act((const float*)y, a.y, a.out_dtype, a.M, a.units, a.stream);
+    if (a.epilogue == TP_EPI_GATED) return tp_gated_act((const float*)y, a.y, a.out_dtype, a.M, a.units, a.act, a.stream);
     return 0;
 }
 
@@ -100,6 +100,8 @@ static int check_args(const GemmArgs& a) {
     if (a.epilogue == TP_EPI_GATED) {
         const int padded = 2 * ((a.units + 15) / 16) * 16;
         TP_REQUIRE(a.units > 0 && a.N == padded, "gated product: %d units need a packed matrix of %d rows, found %d", a.units, padded, a.N);
+        float c1, c3;
+        TP_REQUIRE(tp_gate_constants(a.act, &c1, &c3), "gated product: activation %d is neither gelu-tanh (%d) nor SiLU (%d)", a.act, TP_ACT_GELU_TANH, TP_ACT_SILU);
     }
     return 0;
 }
@@ -139,7 +141,7 @@ static int pick(const GemmArgs& a, int algo) {
 // product comes back as that many K slices
 extern "C" long tp_linear_workspace_bytes(int in_dtype, int out_dtype, int M, int N, int K, int epilogue, int units,
                                           int defer, int algo) {
-    GemmArgs a{nullptr, nullptr, nullptr, in_dtype, out_dtype, M, N, K, epilogue, 1.f, units, nullptr, 0, defer, algo, nullptr};
+    GemmArgs a{nullptr, nullptr, nullptr, in_dtype, out_dtype, M, N, K, epilogue, 1.f, units, 0, nullptr, 0, defer, algo, nullptr};
     const int p = pick(a, algo);
     if (p == 2) return (long)gemm_skinny_workspace(a);
     if (p == 4) return (long)gemv_workspace(a);
@@ -149,9 +151,9 @@ extern "C" long tp_linear_workspace_bytes(int in_dtype, int out_dtype, int M, in
 }
 
 extern "C" int tp_linear(const void* x, const void* w, void* y, int in_dtype, int out_dtype, int M, int N, int K,
-                         int epilogue, float cap, int units, void* workspace, long workspace_bytes, int defer,
+                         int epilogue, float cap, int units, int act, void* workspace, long workspace_bytes, int defer,
                          int algo, void* stream) {
-    GemmArgs a{x, w, y, in_dtype, out_dtype, M, N, K, epilogue, cap, units, workspace, (size_t)workspace_bytes, defer,
+    GemmArgs a{x, w, y, in_dtype, out_dtype, M, N, K, epilogue, cap, units, act, workspace, (size_t)workspace_bytes, defer,
                algo, (hipStream_t)stream};
     if (int rc = check_args(a)) return rc;
     const int p = pick(a, algo);

@@ -38,7 +38,7 @@ __device__ __forceinline__ unsigned in_register(unsigned v) {
 // out in one store where the row length allows the alignment.
 template <int EPI, int TM, int TN>
 __device__ __forceinline__ void store_tile(const f32x4 (&acc)[TM][TN], void* __restrict__ Y, int M, int N, int m0, int n0,
-                                           int wm, int wn, int r, int g, int out_dtype, float cap, int units) {
+                                           int wm, int wn, int r, int g, int out_dtype, float2 epi, int units) {
     const int width = EPI == TP_EPI_GATED ? units : N;
     const bool wide = (width & 3) == 0;
 #pragma unroll
@@ -52,11 +52,11 @@ __device__ __forceinline__ void store_tile(const f32x4 (&acc)[TM][TN], void* __r
             if (EPI == TP_EPI_GATED) {
                 col = ((n0 + wn * 16 * TN + j * 16) >> 1) + g * 4;
 #pragma unroll
-                for (int v = 0; v < 4; v++) o[v] = gelu_tanh_fast(acc[i][j][v]) * acc[i][j + 1 < TN ? j + 1 : j][v];
+                for (int v = 0; v < 4; v++) o[v] = gate_act_fast(acc[i][j][v], epi) * acc[i][j + 1 < TN ? j + 1 : j][v];
             } else {
                 col = n0 + wn * 16 * TN + j * 16 + g * 4;
 #pragma unroll
-                for (int v = 0; v < 4; v++) o[v] = EPI == TP_EPI_SOFTCAP ? softcap_f(acc[i][j][v], cap) : acc[i][j][v];
+                for (int v = 0; v < 4; v++) o[v] = EPI == TP_EPI_SOFTCAP ? softcap_f(acc[i][j][v], epi.x) : acc[i][j][v];
             }
             if (col >= width) continue;
             const size_t at = (size_t)m * width + col;
@@ -86,7 +86,7 @@ __device__ __forceinline__ void store_tile(const f32x4 (&acc)[TM][TN], void* __r
 template <int EPI, int TM, int TN, bool SHORT, int KS = BK>
 __global__ void __launch_bounds__(256, 2)
 gemm_mfma_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __restrict__ Y,
-            int M, int N, int K, int m_tiles, int out_dtype, float cap, int units, int k_per_split, int xcd_panels) {
+            int M, int N, int K, int m_tiles, int out_dtype, float2 epi, int units, int k_per_split, int xcd_panels) {
     constexpr int BM = 32 * TM, BN = 32 * TN, BK = KS, LDS = KS, CPR = KS / 8, LA = TM * KS / 64, LB = TN * KS / 64;
     constexpr int SWZ = CPR >= 16 ? 15 : 7;        // rows 256 bytes long all start at one bank: their 16 chunks are permuted as a whole
     static_assert(!SHORT || KS == 64, "the short load path is written for steps of 64");
@@ -203,7 +203,7 @@ gemm_mfma_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __
         }
     }
 
-    store_tile<EPI, TM, TN>(acc, Y, M, N, m0, n0, wm, wn, r, g, out_dtype, cap, units);
+    store_tile<EPI, TM, TN>(acc, Y, M, N, m0, n0, wm, wn, r, g, out_dtype, epi, units);
 }
 
 // The loop of the large tiles (128 x 128 and 128 x 96) when K is a multiple of 64: the k step's tile comes from
@@ -219,7 +219,7 @@ gemm_mfma_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __
 template <int EPI, int TN>
 __global__ void __launch_bounds__(256, 2)
 gemm_mfma_direct_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __restrict__ Y,
-                   int M, int N, int K, int m_tiles, int out_dtype, float cap, int units, int k_per_split, int xcd_panels) {
+                   int M, int N, int K, int m_tiles, int out_dtype, float2 epi, int units, int k_per_split, int xcd_panels) {
     constexpr int TM = 4, BM = 128, BN = 32 * TN, LDS = BK;
     __shared__ __attribute__((aligned(16))) bf16_t As[BM * LDS];
     __shared__ __attribute__((aligned(16))) bf16_t Bs[BN * LDS];
@@ -298,7 +298,7 @@ gemm_mfma_direct_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, v
         __builtin_amdgcn_s_waitcnt(0);
         __syncthreads();
     }
-    store_tile<EPI, TM, TN>(acc, Y, M, N, m0, n0, wm, wn, r, g, out_dtype, cap, units);
+    store_tile<EPI, TM, TN>(acc, Y, M, N, m0, n0, wm, wn, r, g, out_dtype, epi, units);
 }
 
 bool gemm_mfma_supports(const GemmArgs& a) {
@@ -391,10 +391,10 @@ static void mfma_launch(const GemmArgs& a, void* y, int out_dtype, int splits, i
     const int xcd_panels = (long)m_tiles * n_tiles >= 1024 ? 1 : 0;
     if (TM > 2 && a.M >= 32 * TM && a.N >= 32 * TN)
         gemm_mfma_k<EPI, TM, TN, (TM > 2), KS><<<grid, 256, 0, a.stream>>>((const bf16_t*)a.x, (const bf16_t*)a.w, y, a.M, a.N, a.K, m_tiles,
-                                                                      out_dtype, a.cap, a.units, kps, xcd_panels);
+                                                                      out_dtype, epi_constants(a), a.units, kps, xcd_panels);
     else
         gemm_mfma_k<EPI, TM, TN, false, KS><<<grid, 256, 0, a.stream>>>((const bf16_t*)a.x, (const bf16_t*)a.w, y, a.M, a.N, a.K, m_tiles,
-                                                                   out_dtype, a.cap, a.units, kps, xcd_panels);
+                                                                   out_dtype, epi_constants(a), a.units, kps, xcd_panels);
 }
 
 template <int EPI>
@@ -405,10 +405,10 @@ static void mfma_launch_direct(const GemmArgs& a, Tile t, void* y, int out_dtype
     if (t.tn == 3) {
         if constexpr (EPI != TP_EPI_GATED)
             gemm_mfma_direct_k<EPI, 3><<<grid, 256, 0, a.stream>>>((const bf16_t*)a.x, (const bf16_t*)a.w, y, a.M, a.N, a.K, m_tiles,
-                                                                   out_dtype, a.cap, a.units, kps, xcd_panels);
+                                                                   out_dtype, epi_constants(a), a.units, kps, xcd_panels);
     } else {
         gemm_mfma_direct_k<EPI, 4><<<grid, 256, 0, a.stream>>>((const bf16_t*)a.x, (const bf16_t*)a.w, y, a.M, a.N, a.K, m_tiles,
-                                                               out_dtype, a.cap, a.units, kps, xcd_panels);
+                                                               out_dtype, epi_constants(a), a.units, kps, xcd_panels);
     }
 }
 

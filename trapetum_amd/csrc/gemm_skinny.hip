@@ -33,7 +33,7 @@ __device__ __forceinline__ void store_out(void* y, int out_dtype, size_t idx, fl
 template <int MT, int NT>
 __global__ void __launch_bounds__(256)
 gemm_skinny_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __restrict__ Y, float* __restrict__ part,
-              int M, int N, int K, int k_per_split, int n_splits, int out_dtype, int epilogue, float cap, int units) {
+              int M, int N, int K, int k_per_split, int n_splits, int out_dtype, int epilogue, float2 epi, int units) {
     __shared__ float red[4][MT][64][4];                   // one W tile's partial tiles of the four waves at a time
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
     const int n0 = blockIdx.x * (16 * NT);
@@ -148,7 +148,7 @@ gemm_skinny_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* 
 #pragma unroll
             for (int s = 0; s + 1 < NT; s += 2) {         // tiles alternate: 16 gate rows, the 16 up rows of the same units
                 const int unit = ((n0 + s * 16) >> 1) + nl;
-                if (unit < units) store_out(Y, out_dtype, (size_t)m * units + unit, gelu_tanh_fast(v[t][s]) * v[t][s + 1]);
+                if (unit < units) store_out(Y, out_dtype, (size_t)m * units + unit, gate_act_fast(v[t][s], epi) * v[t][s + 1]);
             }
         } else {
 #pragma unroll
@@ -156,7 +156,7 @@ gemm_skinny_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* 
                 const int n = n0 + s * 16 + nl;
                 if (n >= N) continue;
                 float o = v[t][s];
-                if (epilogue == TP_EPI_SOFTCAP) o = softcap_f(o, cap);
+                if (epilogue == TP_EPI_SOFTCAP) o = softcap_f(o, epi.x);
                 store_out(Y, out_dtype, (size_t)m * N + n, o);
             }
         }
@@ -165,7 +165,7 @@ gemm_skinny_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* 
 
 // adds the K slices in slice order and applies the epilogue
 __global__ void skinny_reduce_k(const float* __restrict__ part, void* __restrict__ Y, int M, int N, int n_splits,
-                                int out_dtype, int epilogue, float cap, int units) {
+                                int out_dtype, int epilogue, float2 epi, int units) {
     const int cols = epilogue == TP_EPI_GATED ? units : N;
     const long total = (long)M * cols;
     for (long idx = blockIdx.x * (long)blockDim.x + threadIdx.x; idx < total; idx += (long)gridDim.x * blockDim.x) {
@@ -178,11 +178,11 @@ __global__ void skinny_reduce_k(const float* __restrict__ part, void* __restrict
                 gsum += p[ng];
                 usum += p[ng + 16];
             }
-            store_out(Y, out_dtype, idx, gelu_tanh_fast(gsum) * usum);
+            store_out(Y, out_dtype, idx, gate_act_fast(gsum, epi) * usum);
         } else {
             float sum = 0.f;
             for (int s = 0; s < n_splits; s++) sum += part[((size_t)s * M + m) * N + c];
-            if (epilogue == TP_EPI_SOFTCAP) sum = softcap_f(sum, cap);
+            if (epilogue == TP_EPI_SOFTCAP) sum = softcap_f(sum, epi.x);
             store_out(Y, out_dtype, idx, sum);
         }
     }
@@ -224,13 +224,13 @@ template <int MT>
 static void launch_mt(const GemmArgs& a, int nt, dim3 grid, float* part, int kps, int splits) {
     if (nt == 4)
         gemm_skinny_k<MT, 4><<<grid, 256, 0, a.stream>>>((const bf16_t*)a.x, (const bf16_t*)a.w, a.y, part, a.M, a.N, a.K,
-                                                         kps, splits, a.out_dtype, a.epilogue, a.cap, a.units);
+                                                         kps, splits, a.out_dtype, a.epilogue, epi_constants(a), a.units);
     else if (nt == 2)
         gemm_skinny_k<MT, 2><<<grid, 256, 0, a.stream>>>((const bf16_t*)a.x, (const bf16_t*)a.w, a.y, part, a.M, a.N, a.K,
-                                                         kps, splits, a.out_dtype, a.epilogue, a.cap, a.units);
+                                                         kps, splits, a.out_dtype, a.epilogue, epi_constants(a), a.units);
     else
         gemm_skinny_k<MT, 1><<<grid, 256, 0, a.stream>>>((const bf16_t*)a.x, (const bf16_t*)a.w, a.y, part, a.M, a.N, a.K,
-                                                         kps, splits, a.out_dtype, a.epilogue, a.cap, a.units);
+                                                         kps, splits, a.out_dtype, a.epilogue, epi_constants(a), a.units);
 }
 
 int gemm_skinny_launch(const GemmArgs& a) {
@@ -253,7 +253,7 @@ int gemm_skinny_launch(const GemmArgs& a) {
         const long total = (long)a.M * (a.epilogue == TP_EPI_GATED ? a.units : a.N);
         int rb = tp_cdiv(total, 256);
         if (rb > 2048) rb = 2048;
-        skinny_reduce_k<<<rb, 256, 0, a.stream>>>(part, a.y, a.M, a.N, splits, a.out_dtype, a.epilogue, a.cap, a.units);
+        skinny_reduce_k<<<rb, 256, 0, a.stream>>>(part, a.y, a.M, a.N, splits, a.out_dtype, a.epilogue, epi_constants(a), a.units);
         return tp_check_launch("linear (skinny reduce)");
     }
     return 0;

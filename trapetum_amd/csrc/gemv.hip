@@ -24,7 +24,7 @@ __device__ __forceinline__ float hi_f32(uint32_t pair) { return __uint_as_float(
 template <int MR, int NC>
 __global__ void __launch_bounds__(256)
 gemv_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __restrict__ Y, float* __restrict__ part,
-       int M, int N, int K, int k_per_split, int n_splits, int out_dtype, int epilogue, float cap, int units) {
+       int M, int N, int K, int k_per_split, int n_splits, int out_dtype, int epilogue, float2 epi, int units) {
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int kbeg = blockIdx.y * k_per_split, klen = min(K, kbeg + k_per_split) - kbeg;
     // a chunk past the slice reads the slice's first elements (loads stay unconditional) against X values of zero
@@ -91,7 +91,7 @@ gemv_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __restr
                 if (row[j] < N) part[((size_t)blockIdx.y * M + m) * N + row[j]] = acc[j][m];
         } else if (epilogue == TP_EPI_GATED) {
             if (item < units) {
-                const float o = gelu_tanh_fast(acc[0][m]) * acc[1][m];
+                const float o = gate_act_fast(acc[0][m], epi) * acc[1][m];
                 if (out_dtype == TP_F32) ((float*)Y)[(size_t)m * units + item] = o;
                 else ((bf16_t*)Y)[(size_t)m * units + item] = f32_to_bf16(o);
             }
@@ -100,7 +100,7 @@ gemv_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __restr
             for (int j = 0; j < GV_ROWS; j++) {
                 if (row[j] >= N) continue;
                 float o = acc[j][m];
-                if (epilogue == TP_EPI_SOFTCAP) o = softcap_f(o, cap);
+                if (epilogue == TP_EPI_SOFTCAP) o = softcap_f(o, epi.x);
                 if (out_dtype == TP_F32) ((float*)Y)[(size_t)m * N + row[j]] = o;
                 else ((bf16_t*)Y)[(size_t)m * N + row[j]] = f32_to_bf16(o);
             }
@@ -132,7 +132,7 @@ size_t gemv_workspace(const GemmArgs& a) {
 template <int MR, int NC>
 static void gemv_launch_nc(const GemmArgs& a, dim3 grid, float* part, int kps, int splits) {
     gemv_k<MR, NC><<<grid, 256, 0, a.stream>>>((const bf16_t*)a.x, (const bf16_t*)a.w, a.y, part, a.M, a.N, a.K, kps, splits,
-                                              a.out_dtype, a.epilogue, a.cap, a.units);
+                                              a.out_dtype, a.epilogue, epi_constants(a), a.units);
 }
 
 template <int MR>

@@ -20,7 +20,10 @@ class AssembledLayer:
         mixer = build_part("mixer", lspec.mixer)
         ff = build_part("feed_forward", lspec.feed_forward)
         block_cls = part_class("block", lspec.block[0])
-        self.block = block_cls(mixer, ff, lambda: build_part("norm", lspec.norm), **lspec.block[1])
+        unknown = set(lspec.norms or {}) - set(block_cls.norm_sites())
+        if unknown:
+            raise ValueError(f"the layer's spec names norms for {sorted(unknown)}, block '{lspec.block[0]}' has {list(block_cls.norm_sites())}")
+        self.block = block_cls(mixer, ff, lambda site: build_part("norm", lspec.norm_of(site)), **lspec.block[1])
         self.prefixes = lspec.prefixes
         self.places = [(mixer, self._prefix("mixer")), (ff, self._prefix("feed_forward"))]
         for site, norm in self.block.norms.items():

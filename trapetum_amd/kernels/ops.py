@@ -22,8 +22,8 @@ _CORE_SIGS = {
     "tp_rope_kv_write": [_P, _L, _P, _L, _P, _L, _I, _I, _I, _I, _I, _P, _I, _P, _P, _P, _P, _I, _P, _P, _I, _I,
                          _P, _P, _L, _P, _P],
     "tp_gather_kv_prefix": [_P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P, _P, _P, _I, _P, _P, _L, _P],
-    "tp_gated_act": [_P, _P, _I, _I, _I, _P],
-    "tp_linear": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P, _L, _I, _I, _P],
+    "tp_gated_act": [_P, _P, _I, _I, _I, _I, _P],
+    "tp_linear": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P, _L, _I, _I, _P],
     "tp_linear_workspace_bytes": [_I, _I, _I, _I, _I, _I, _I, _I, _I],
     "tp_attn_simple_prefill": [_P, _L, _P, _L, _P, _L, _I, _I, _I, _I, _I, _P, _P, _P, _F, _F, _I, _P, _P],
     "tp_attn_simple_decode": [_P, _L, _I, _I, _I, _I, _I, _P, _P, _I, _P, _P, _I, _I, _F, _F, _I, _P, _P],
@@ -44,6 +44,7 @@ _ATTN_SIGS = {
 }
 
 EPI_NONE, EPI_SOFTCAP, EPI_GATED = 0, 1, 2
+GATE_ACTIVATIONS = {"gelu_tanh": 0, "silu": 1}       # what a gated product's epilogue can apply to the gate
 GATE_GROUP = 16
 
 
@@ -279,7 +280,7 @@ class HipOps:
         return gk, gv
 
     # ---- matrix products -----------------------------------------------------------------------------
-    def _linear(self, x, w, out_dtype, epilogue, cap, units, defer=False):
+    def _linear(self, x, w, out_dtype, epilogue, cap, units, defer=False, act=0):
         self._dev(x, w)
         if x.dim() != 2 or w.dim() != 2 or not x.is_contiguous() or not w.is_contiguous():
             raise KernelError("linear: rows and matrix must be contiguous 2-D tensors")
@@ -296,12 +297,12 @@ class HipOps:
         if defer and epilogue == EPI_NONE and nbytes and nbytes % (m * n * 4) == 0 and nbytes // (m * n * 4) > 1:
             slices = torch.empty((nbytes // (m * n * 4), m, n), dtype=torch.float32, device=self.device)
             self._call(self.lib, "tp_linear", x.data_ptr(), w.data_ptr(), None, _code(x.dtype), _code(out_dtype),
-                       m, n, k, epilogue, float(cap), units, slices.data_ptr(), nbytes, 1, algo, self._stream())
+                       m, n, k, epilogue, float(cap), units, act, slices.data_ptr(), nbytes, 1, algo, self._stream())
             return SplitRows(slices)
         out = torch.empty((m, cols), dtype=out_dtype, device=self.device)
         ws = torch.empty(nbytes, dtype=torch.uint8, device=self.device) if nbytes else None
         self._call(self.lib, "tp_linear", x.data_ptr(), w.data_ptr(), out.data_ptr(), _code(x.dtype), _code(out_dtype),
-                   m, n, k, epilogue, float(cap), units, ws.data_ptr() if ws is not None else None, nbytes, 0, algo,
+                   m, n, k, epilogue, float(cap), units, act, ws.data_ptr() if ws is not None else None, nbytes, 0, algo,
                    self._stream())
         return out
 
@@ -313,9 +314,10 @@ class HipOps:
         return self._linear(x, w, out_dtype, EPI_NONE, 0.0, 0, defer=defer)
 
     def gated_linear(self, x, w_packed, inter, activation, out_dtype):
-        if activation != "gelu_tanh":
-            raise KernelError(f"gated_linear: activation '{activation}' has no kernel (gelu_tanh)")
-        return self._linear(x, w_packed, out_dtype, EPI_GATED, 0.0, inter)
+        """act(x @ gate^T) * (x @ up^T) over the packed matrix of `pack_gate_up`; activation: one of GATE_ACTIVATIONS."""
+        if activation not in GATE_ACTIVATIONS:
+            raise KernelError(f"gated_linear: activation '{activation}' has no kernel ({', '.join(GATE_ACTIVATIONS)})")
+        return self._linear(x, w_packed, out_dtype, EPI_GATED, 0.0, inter, act=GATE_ACTIVATIONS[activation])
 
     # ---- attention -------------------------------------------------------------------------------------
     def _fast_attention(self, dtype, H, KV, hd):

@@ -25,8 +25,12 @@ class LayerSpec:
     block: PartRef
     mixer: PartRef
     feed_forward: PartRef
-    norm: PartRef                    # built once for every norm site the block declares
+    norm: PartRef                    # built once for every norm site the block declares ...
     prefixes: Dict[str, str]         # site name of the block -> checkpoint prefix
+    norms: Optional[Dict[str, PartRef]] = None    # ... unless a site is named here with a norm of its own
+
+    def norm_of(self, site):
+        return (self.norms or {}).get(site, self.norm)
 
 
 @dataclasses.dataclass

@@ -64,9 +64,10 @@ class FeedForward(Part):
 
 class Block(Part):
     def __init__(self, mixer, feed_forward, make_norm):
+        """make_norm(site) builds the norm that stands at one of the block's sites."""
         self.mixer = mixer
         self.feed_forward = feed_forward
-        self.norms = {name: make_norm() for name in self.norm_sites()}
+        self.norms = {name: make_norm(name) for name in self.norm_sites()}
 
     @classmethod
     def norm_sites(cls):
