@@ -74,3 +74,22 @@ def test_float32_weights_are_kept_as_drawn(tmp_path):
     assert rel_l2(got, plain.forward(pcfg, pw, toks)) < 1e-5
     rounded = {k: v.float().to(torch.bfloat16).double() for k, v in pw.items()}
     assert rel_l2(got, plain.forward(pcfg, rounded, toks)) > 1e-4
+
+
+def test_switches(tmp_path):
+    """TRAPETUM_AMD_PROFILE=1 prints the time per entry point of the kernel library when the process ends;
+    TRAPETUM_AMD_FORCE_PLAIN=1 runs bfloat16 on the plain kernels, with the same tokens where the model is sure."""
+    config = tmp_path / "config.json"
+    config.write_text(json.dumps(dict(TINY_A, architectures=["Gemma2ForCausalLM"])))
+    args = [sys.executable, "-m", "trapetum_amd", "run", "--random", str(config), "--prompt-ids", "5,6,7,8", "--max-tokens", "6",
+            "--no-stop"]
+    p = subprocess.run(args, cwd=ROOT, capture_output=True, text=True, timeout=300, env=dict(os.environ, TRAPETUM_AMD_PROFILE="1"))
+    assert p.returncode == 0, p.stderr[-2000:]
+    prof = [l for l in p.stderr.splitlines() if l.startswith("[profile] op=")]
+    ops = {l.split()[1][3:]: int(l.split()[2][6:]) for l in prof}
+    assert ops["tp_linear"] > 0 and ops["tp_add_rms_norm"] > 0 and "tp_attn_decode_fused" in ops, p.stderr[-2000:]
+    ids = p.stdout.strip()
+    p = subprocess.run(args, cwd=ROOT, capture_output=True, text=True, timeout=300, env=dict(os.environ, TRAPETUM_AMD_FORCE_PLAIN="1", TRAPETUM_AMD_PROFILE="1"))
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert "tp_attn_decode_fused" not in p.stderr and "tp_attn_simple_decode" in p.stderr
+    assert p.stdout.strip() == ids

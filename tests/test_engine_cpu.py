@@ -83,3 +83,36 @@ def test_portions_and_joining_requests(setup, page_size):
         assert cache.live_slots() == []
         for rid in requests:
             assert rel_l2(torch.from_numpy(got[rid]), ref[rid]) < 2e-5, rid
+
+
+def test_debug_dump_lines(setup, monkeypatch, capsys):
+    """TRAPETUM_AMD_DEBUG_DUMP=1: one `[ldump]` line per layer and stage in the reference's format
+    (runtime/src/lib.rs:1384-1389), the statistics being those of the step's rows, and the five largest logits."""
+    import re
+
+    from trapetum_amd import flags
+    model, cfg, pcfg, pw = setup
+    toks = random_tokens(9, cfg.vocab_size, 8)
+    monkeypatch.setenv("TRAPETUM_AMD_DEBUG_DUMP", "1")
+    flags._on.cache_clear()
+    try:
+        cache = model.new_cache(max_tokens=64)
+        s = cache.acquire()
+        logits = model.step(cache, [s], toks, counts=[9], want=[8])
+    finally:
+        monkeypatch.delenv("TRAPETUM_AMD_DEBUG_DUMP")
+        flags._on.cache_clear()
+    lines = [l for l in capsys.readouterr().err.splitlines() if l.startswith("[ldump]")]
+    pattern = re.compile(r"^\[ldump\] L=(-?\d+) stage=(\w+) l2=(\S+) absmax=(\S+) mean=(\S+)$")
+    rows = [pattern.match(l).groups() for l in lines[:-1]]
+    stages = ["mixer_in", "mixer_out", "after_mixer", "ff_out", "layer_out"]
+    assert [(int(r[0]), r[1]) for r in rows] == [(-1, "embed")] + [(l, st) for l in range(cfg.num_hidden_layers) for st in stages] \
+        + [(-1, "final_norm"), (-1, "logits")]
+    assert abs(float(rows[-1][2]) - float(logits.double().norm())) < 1e-4 * float(logits.double().norm())
+    x = plain.embed(torch.tensor(toks), pw["model.embed_tokens.weight"], cfg.hidden_size)
+    assert abs(float(rows[0][3]) - float(x.abs().max())) < 1e-5 * float(x.abs().max())
+    top = lines[-1]
+    assert top.startswith("[ldump] top5= ") and int(top.split()[2].split(":")[0]) == int(logits[0].argmax())
+    # switched off, nothing is printed
+    model.step(cache, [s], [toks[0]])
+    assert "[ldump]" not in capsys.readouterr().err

@@ -165,6 +165,17 @@ class StepContext:
     def page_table(self, group_index):
         return self._tables[group_index]
 
+    def dump(self, stage, x):
+        """With TRAPETUM_AMD_DEBUG_DUMP=1: one line of statistics of `x` (rows of the step at this stage of the running
+        schedule entry) on stderr; nothing otherwise."""
+        from .. import flags
+        if not flags.debug_dump() or x is None:
+            return
+        import sys
+        t = self.ops.rows(x, x.dtype).double()
+        print(f"[ldump] L={-1 if self.entry is None else self.entry} stage={stage} l2={float(t.norm()):.6e} "
+              f"absmax={float(t.abs().max()):.6e} mean={float(t.mean()):.6e}", file=sys.stderr, flush=True)
+
     def keys_of(self, group_index):
         """The KeyGeometry of a cache group in an "extend" step (host arrays, and `*_dev` int32 on the device)."""
         return self.key_geometry[group_index]

@@ -53,7 +53,8 @@ class Engine:
             max_context = min(max_tokens_in_cache, limit) if limit else max_tokens_in_cache
         self.cache = model.new_cache(max_tokens_in_cache, max_context=max_context, max_slots=max_batch, page_size=page_size)
         self.graphed = None
-        if use_graph and model.rt.device.type == "cuda":
+        from .. import flags
+        if use_graph and model.rt.device.type == "cuda" and flags.graphs_allowed():
             from .graphs import GraphedDecode
             self.graphed = GraphedDecode(model, self.cache)
 

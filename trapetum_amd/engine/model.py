@@ -155,6 +155,7 @@ class Model:
         ctx.mark_shared(self._shared)
         cache = ctx.cache
         stream = self.embedding.forward(ctx, tok)
+        ctx.dump("embed", stream)
         whole = ctx.n_want == ctx.n_rows and ctx.identity_want
         normed = None
         last = len(self.schedule) - 1
@@ -177,4 +178,14 @@ class Model:
         else:
             rows = stream if whole else ctx.ops.gather_rows(stream, ctx.want_rows)
             rows = self.final_norm.forward(ctx, rows)
-        return self.head.forward(ctx, rows)
+        ctx.entry = None
+        ctx.dump("final_norm", rows)
+        logits = self.head.forward(ctx, rows)
+        ctx.dump("logits", logits)
+        from .. import flags
+        if flags.debug_dump():                  # the five largest logits of the last wanted row, smaller ids first on ties
+            import sys
+            z = logits[-1].double().cpu()
+            order = sorted(range(z.numel()), key=lambda i: (-float(z[i]), i))[:5]
+            print("[ldump] top5= " + ",".join(f"{i}:{float(z[i]):.4f}" for i in order), file=sys.stderr, flush=True)
+        return logits

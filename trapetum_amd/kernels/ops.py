@@ -93,17 +93,46 @@ class HipOps:
         _bind(self.lib, _CORE_SIGS)
         self._attn = {}
         self._sample_ws = {}
-        self.force_linear = 0           # tests: 1 plain, 2 skinny, 3 tiled (6: its wide tile, 7: its 128 x 96 tile, 8, 9: loads into LDS, 128 x 128 and 128 x 96), 4 multiply-adds (1-2 rows)
-        self.force_plain_attention = False
+        from .. import flags
+        plain = flags.force_plain()
+        self.force_linear = 1 if plain else 0   # 1 plain, 2 skinny, 3 tiled (6: its wide tile, 7: its 128 x 96 tile, 8, 9: loads into LDS, 128 x 128 and 128 x 96), 4 multiply-adds (1-2 rows)
+        self.force_plain_attention = plain
+        self._timed = None                      # with TRAPETUM_AMD_PROFILE=1: [(entry point, start event, end event)]
+        if flags.profile():
+            import atexit
+            self._timed = []
+            atexit.register(self.profile_report)
 
     # ---- helpers -----------------------------------------------------------------------------------
     def _stream(self):
         return torch.cuda.current_stream(self.device).cuda_stream
 
     def _call(self, lib, name, *args):
-        rc = getattr(lib, name)(*args)
+        if self._timed is not None:
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            rc = getattr(lib, name)(*args)
+            b.record()
+            self._timed.append((name, a, b))
+        else:
+            rc = getattr(lib, name)(*args)
         if rc != 0:
             raise KernelError(lib.tp_last_error().decode())
+
+    def profile_report(self, file=None):
+        """The time of the calls so far per entry point, most expensive first (TRAPETUM_AMD_PROFILE=1); forgets them."""
+        import sys
+        if not self._timed:
+            return
+        torch.cuda.synchronize(self.device)
+        total = {}
+        for name, a, b in self._timed:
+            ms, n = total.get(name, (0.0, 0))
+            total[name] = (ms + a.elapsed_time(b), n + 1)
+        self._timed = []
+        out = file or sys.stderr
+        for name, (ms, n) in sorted(total.items(), key=lambda kv: -kv[1][0]):
+            print(f"[profile] op={name} calls={n} total_ms={ms:.3f} mean_us={1e3 * ms / n:.2f}", file=out, flush=True)
 
     def _dev(self, *tensors):
         for t in tensors:

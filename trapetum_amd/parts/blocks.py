@@ -41,10 +41,16 @@ class SandwichBlock(Block):
     def forward(self, ctx, stream, site, normed=None, next_norm=None):
         n = self.norms
         x = normed if normed is not None else n["pre_mixer_norm"].forward(ctx, stream)
+        ctx.dump("mixer_in", x)
         a = self.mixer.forward(ctx, x, site)
+        ctx.dump("mixer_out", a)
         x = add_then_norm(ctx, stream, a, n["post_mixer_norm"], n["pre_ff_norm"])
+        ctx.dump("after_mixer", stream)
         m = self.feed_forward.forward(ctx, x)
-        return stream, add_then_norm(ctx, stream, m, n["post_ff_norm"], next_norm)
+        ctx.dump("ff_out", m)
+        normed_next = add_then_norm(ctx, stream, m, n["post_ff_norm"], next_norm)
+        ctx.dump("layer_out", stream)
+        return stream, normed_next
 
 
 class PreNormBlock(Block):
@@ -58,10 +64,16 @@ class PreNormBlock(Block):
     def forward(self, ctx, stream, site, normed=None, next_norm=None):
         n = self.norms
         x = normed if normed is not None else n["pre_mixer_norm"].forward(ctx, stream)
+        ctx.dump("mixer_in", x)
         a = self.mixer.forward(ctx, x, site)
+        ctx.dump("mixer_out", a)
         x = add_then_norm(ctx, stream, a, None, n["pre_ff_norm"])
+        ctx.dump("after_mixer", stream)
         m = self.feed_forward.forward(ctx, x)
-        return stream, add_then_norm(ctx, stream, m, None, next_norm)
+        ctx.dump("ff_out", m)
+        normed_next = add_then_norm(ctx, stream, m, None, next_norm)
+        ctx.dump("layer_out", stream)
+        return stream, normed_next
 
 
 register_part("block", "sandwich", SandwichBlock)
