@@ -69,7 +69,8 @@ def test_add_rms_norm(ops, dt, post, nxt, m, d):
 
 
 @pytest.mark.parametrize("m,n,k", [(8, 2304, 2048), (3, 600, 9216), (64, 2304, 4096), (700, 2304, 2048), (300, 520, 4104),
-                                   (2048, 2304, 4096), (1, 2304, 9216), (2, 601, 14336)])
+                                   (2048, 2304, 4096), (1, 2304, 9216), (2, 601, 14336),
+                                   (5, 2304, 9216), (8, 77, 1544), (4, 4608, 4096), (7, 1000, 20000)])
 def test_deferred_product_into_add_rms_norm(ops, m, n, k):
     """A product left in K slices and added by add_rms_norm equals the product, then the norm."""
     from trapetum_amd.kernels.ops import SplitRows
@@ -129,7 +130,12 @@ LINEAR_SHAPES += [(300, 44177, 64), (40, 70001, 72)]
 LINEAR_SHAPES += [(1, 77, 8), (2, 301, 1000), (2, 130, 1536), (1, 257, 3584), (2, 99, 4608), (1, 64, 5120)]
 
 
-@pytest.mark.parametrize("algo", [1, 2, 3, 4, 6, 7, 8, 9])
+# three to eight rows, for the kernel of blocks of 8 rows of W: an N that is no multiple of 8 or 16, a K that ends inside a
+# step of 64, inside a wave's quarter and in a second round of loads, every number of rows of X
+LINEAR_SHAPES += [(3, 77, 8), (8, 1001, 2304), (7, 130, 2312), (6, 250, 5000), (4, 4099, 600), (5, 9, 9216)]
+
+
+@pytest.mark.parametrize("algo", [1, 2, 3, 4, 5, 6, 7, 8, 9])
 @pytest.mark.parametrize("m,n,k", LINEAR_SHAPES)
 def test_linear_bf16(ops, algo, m, n, k):
     if algo in (8, 9) and k % 64:
@@ -138,6 +144,8 @@ def test_linear_bf16(ops, algo, m, n, k):
         pytest.skip("the skinny kernel takes at most 64 rows")
     if algo == 4 and (m > 2 or k > 5120):
         pytest.skip("the multiply-add kernel takes at most 2 rows and, unsliced, a K of 5120")
+    if algo == 5 and m > 8:
+        pytest.skip("the kernel of 8-row blocks takes at most 8 rows")
     x, w = randn(m, k, dtype=torch.bfloat16, seed=7), randn(n, k, dtype=torch.bfloat16, seed=8, scale=0.05)
     ops.force_linear = algo
     try:
@@ -163,15 +171,18 @@ def test_linear_f32(ops, m, n, k):
     assert torch.equal(alone[0], got[m - 1])
 
 
-@pytest.mark.parametrize("algo", [1, 2, 3, 4, 6, 8])
+@pytest.mark.parametrize("algo", [1, 2, 3, 4, 5, 6, 8])
 @pytest.mark.parametrize("dt", ["bf16", "f32"])
 @pytest.mark.parametrize("m,inter,k", [(1, 16, 16), (4, 200, 88), (40, 320, 96), (9, 1000, 2304), (150, 72, 136),
-                                       (150, 72, 128), (700, 1000, 320), (130, 36010, 64), (2, 1000, 2304), (1, 75, 4608)])
+                                       (150, 72, 128), (700, 1000, 320), (130, 36010, 64), (2, 1000, 2304), (1, 75, 4608),
+                                       (8, 9216, 2304), (3, 41, 2504), (7, 8, 520)])
 def test_gated_linear(ops, algo, dt, m, inter, k):
     if dt == "f32" and algo != 1:
         pytest.skip("float32 runs on the plain kernel only")
     if algo == 4 and m > 2:
         pytest.skip("the multiply-add kernel takes at most 2 rows")
+    if algo == 5 and m > 8:
+        pytest.skip("the kernel of 8-row blocks takes at most 8 rows")
     if algo == 2 and m > 64:
         pytest.skip("the skinny kernel takes at most 64 rows")
     if algo in (8, 9) and k % 64:
@@ -194,7 +205,7 @@ def test_gated_linear(ops, algo, dt, m, inter, k):
     assert rel_l2(silu, torch.nn.functional.silu(g) * u) < (5e-6 if dt == "f32" else 4e-3)      # the other activation offered
 
 
-@pytest.mark.parametrize("algo,m", [(2, 8), (3, 8), (3, 200)])
+@pytest.mark.parametrize("algo,m", [(2, 8), (3, 8), (3, 200), (5, 8), (5, 3)])
 def test_gated_linear_at_the_ends_of_the_activation(ops, algo, m):
     """Gate values far out on both sides (the activation is the identity on one, zero on the other): no overflow of the
     exponential shows in the result."""

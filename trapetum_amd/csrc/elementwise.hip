@@ -219,16 +219,21 @@ add_rms_norm_vec_k(float* __restrict__ stream, const TR* __restrict__ rows, int 
         const int i = (threadIdx.x + j * NTH) * 4;
         const bool ok = i < D;
         const int ic = ok ? i : 0;                       // a chunk past the row reads the row's first and counts as zero
-        ld4(ar + ic, a[j]);
-        for (int sl = 1; sl < n_slices; sl++) {          // slices in slice order
-            float t[4];
-            ld4(ar + (size_t)sl * slice_stride + ic, t);
-#pragma unroll
-            for (int e = 0; e < 4; e++) a[j][e] += t[e];
-        }
+        // the stream, the gains and up to four slices are asked for together: a loop of load-then-add would pay one
+        // trip to memory per slice.  Slices are added in slice order; past the last one the load repeats it and adds nothing.
         ld4(sr + ic, v[j]);
         if (gain_post) ld4(gain_post + ic, gp[j]);
         if (gain_next) ld4(gain_next + ic, gn[j]);
+        ld4(ar + ic, a[j]);
+        for (int s0 = 1; s0 < n_slices; s0 += 4) {
+            float t[4][4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) ld4(ar + (size_t)(s0 + u < n_slices ? s0 + u : n_slices - 1) * slice_stride + ic, t[u]);
+#pragma unroll
+            for (int u = 0; u < 4; u++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) a[j][e] += s0 + u < n_slices ? t[u][e] : 0.f;
+        }
 #pragma unroll
         for (int e = 0; e < 4; e++) {
             if (!ok) { a[j][e] = 0.f; v[j][e] = 0.f; }

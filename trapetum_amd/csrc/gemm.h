@@ -35,6 +35,10 @@ int gemm_skinny_launch(const GemmArgs& a);
 bool gemv_supports(const GemmArgs& a);
 size_t gemv_workspace(const GemmArgs& a);
 int gemv_launch(const GemmArgs& a);
+// bf16 on the matrix cores for three to eight rows: blocks of 8 rows of W, every load of a block in flight at once
+bool gemm_rows8_supports(const GemmArgs& a);
+size_t gemm_rows8_workspace(const GemmArgs& a);
+int gemm_rows8_launch(const GemmArgs& a);
 bool gemm_mfma_supports(const GemmArgs& a);
 int gemm_mfma_splits(const GemmArgs& a);
 int gemm_mfma_launch(const GemmArgs& a);

@@ -107,10 +107,12 @@ static int check_args(const GemmArgs& a) {
 }
 
 // algo: 0 = choose, 1 = plain, 2 = skinny matrix-core, 3 = tiled matrix-core (6: with its wide tile, 7: with its 128 x 96 tile,
-// 8, 9: with its loop that loads straight into LDS, 128 x 128 and 128 x 96), 4 = multiply-adds for one or two rows
+// 8, 9: with its loop that loads straight into LDS, 128 x 128 and 128 x 96), 4 = multiply-adds for one or two rows,
+// 5 = matrix-core kernel for up to eight rows
 static int pick(const GemmArgs& a, int algo) {
     if (algo == 1) return 1;
     if (algo == 4) return gemv_supports(a) ? 4 : -4;
+    if (algo == 5) return gemm_rows8_supports(a) ? 5 : -5;
     if (algo == 2) return gemm_skinny_supports(a) ? 2 : -2;
     if (algo == 3 || algo == 6 || algo == 7 || algo == 8 || algo == 9) return gemm_mfma_supports(a) ? 3 : -3;
     // Up to 64 rows both matrix-core kernels stream W once; which is faster was measured on MI355X at the 2B shapes
@@ -121,6 +123,24 @@ static int pick(const GemmArgs& a, int algo) {
     //   o       N 2304  K 2048      8 rows  5.2 /  5.5   32 rows  7.7 /  6.0   64 rows 13.3 /  6.7   (K slices)
     //   gate/up N 18432 K 2304      8 rows 26.9 / 24.2   32 rows 40.7 / 24.7   64 rows 48.5 / 26.5   (no slices: gated)
     if (gemv_supports(a)) return 4;          // one or two rows: 2B gate/up 16.8 against 22.6 us on the skinny kernel
+    // Three to eight rows: the kernel whose blocks read 8 rows of W in one go, where it was measured faster than the
+    // choice below (microseconds from a replayed graph, cold weights, that choice / this kernel / a kernel that only reads):
+    //   2B  gate/up 24.1 / 21.7 / 15.2   down 14.5 / 11.5 / 9.1   qkv 7.1 / 6.3 / 4.9   o 5.0 / 5.2 / 4.2   logits 209 / 253 / 204
+    //   9B  gate/up 43.2 / 45.6 / 36.1   down 22.0 / 24.5 / 18.6  qkv 13.5 / 15.1 / 12.1  o 10.0 / 9.2 / 7.6
+    //   27B gate/up 141 / 136 / 116      down 72.4 / 76.7 / 58.2  qkv 16.8 / 19.9 / 14.9  o 14.5 / 10.8 / 8.3   logits 407 / 462 / 414
+    // at 8 rows; at 3 and 4 rows, where the choice below is the skinny kernel, 2B logits 250 / 228, 9B gate/up 49.3 / 41.8,
+    // 27B gate/up 142 / 127, 27B qkv 16.9 / 19.4.  A slice of K beyond 2,304 takes the kernel a second round of loads.
+    // A decode step of 8 sequences at the 2B sizes: 2.30 -> 2.00 ms.
+    if (a.M <= 8 && gemm_rows8_supports(a)) {
+        const long nk = (long)a.N * a.K;
+        if (a.defer && a.epilogue == TP_EPI_NONE) {
+            if (nk <= 32000000) return 5;     // (2B o alone is no faster, 5.0 / 5.2, but a step of 8 sequences is: 2.001 -> 1.988 ms)
+        } else if (a.M < 8) {
+            if (a.epilogue == TP_EPI_GATED || a.K <= 2304 || a.N >= 32768) return 5;
+        } else if (a.K <= 2304 && a.N < 32768) {
+            return 5;
+        }
+    }
     if (gemm_mfma_supports(a)) {
         const bool sliced = a.defer && a.epilogue == TP_EPI_NONE;
         // (up to 16 rows the tiled kernel's lead on qkv and down is lost again in their consumers, which then add
@@ -145,6 +165,7 @@ extern "C" long tp_linear_workspace_bytes(int in_dtype, int out_dtype, int M, in
     const int p = pick(a, algo);
     if (p == 2) return (long)gemm_skinny_workspace(a);
     if (p == 4) return (long)gemv_workspace(a);
+    if (p == 5) return (long)gemm_rows8_workspace(a);
     if (p == 3) { const int s = gemm_mfma_splits(a); return s > 1 ? (long)s * M * N * 4 : 0; }
     if (p == 1 && epilogue == TP_EPI_GATED) return (long)M * N * 4;
     return 0;
@@ -160,6 +181,7 @@ extern "C" int tp_linear(const void* x, const void* w, void* y, int in_dtype, in
     TP_REQUIRE(p > 0, "linear: the requested kernel (%d) does not take M=%d N=%d K=%d dtype %d", algo, M, N, K, in_dtype);
     if (p == 2) return gemm_skinny_launch(a);
     if (p == 4) return gemv_launch(a);
+    if (p == 5) return gemm_rows8_launch(a);
     if (p == 3) return gemm_mfma_launch(a);
     return gemm_simple_launch(a);
 }

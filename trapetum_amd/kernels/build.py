@@ -18,7 +18,7 @@ CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))),
 ARCH = "gfx950"
 FLAGS = ["--offload-arch=" + ARCH, "-O3", "-fPIC", "-std=c++17",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-result"]
-CORE_SOURCES = ["elementwise.hip", "gemm.hip", "gemm_skinny.hip", "gemm_mfma.hip", "gemv.hip", "attention_simple.hip", "sampling.hip", "probes.hip"]
+CORE_SOURCES = ["elementwise.hip", "gemm.hip", "gemm_skinny.hip", "gemm_mfma.hip", "gemv.hip", "gemm_rows8.hip", "attention_simple.hip", "sampling.hip", "probes.hip"]
 ATTN_SOURCE = "attention_mfma.hip"
 _NOISE = "is not a recognized feature for this target"
 
