@@ -1,6 +1,7 @@
 // Row-wise kernels: embedding, norms fused with the residual add, row gather, RoPE + cache write,
 // gated activation.  One block per row; statistics, angles and sums in fp32.
 #include "common.h"
+#include <type_traits>
 
 #include "error_channel.h"
 
@@ -219,21 +220,28 @@ add_rms_norm_vec_k(float* __restrict__ stream, const TR* __restrict__ rows, int 
         const int i = (threadIdx.x + j * NTH) * 4;
         const bool ok = i < D;
         const int ic = ok ? i : 0;                       // a chunk past the row reads the row's first and counts as zero
-        // the stream, the gains and up to four slices are asked for together: a loop of load-then-add would pay one
-        // trip to memory per slice.  Slices are added in slice order; past the last one the load repeats it and adds nothing.
+        // the stream, the gains and a group of slices are asked for together: a loop of load-then-add would pay one
+        // trip to memory per slice.  Slices are added in slice order; past the last one the load repeats it and adds
+        // nothing.  Groups of four; a row of one chunk a lane takes twelve at a time while more than four are left
+        // (a product of few rows comes in up to sixteen slices).
         ld4(sr + ic, v[j]);
         if (gain_post) ld4(gain_post + ic, gp[j]);
         if (gain_next) ld4(gain_next + ic, gn[j]);
         ld4(ar + ic, a[j]);
-        for (int s0 = 1; s0 < n_slices; s0 += 4) {
-            float t[4][4];
+        auto add_group = [&](int s0, auto width) {
+            constexpr int W = decltype(width)::value;
+            float t[W][4];
 #pragma unroll
-            for (int u = 0; u < 4; u++) ld4(ar + (size_t)(s0 + u < n_slices ? s0 + u : n_slices - 1) * slice_stride + ic, t[u]);
+            for (int u = 0; u < W; u++) ld4(ar + (size_t)(s0 + u < n_slices ? s0 + u : n_slices - 1) * slice_stride + ic, t[u]);
 #pragma unroll
-            for (int u = 0; u < 4; u++)
+            for (int u = 0; u < W; u++)
 #pragma unroll
                 for (int e = 0; e < 4; e++) a[j][e] += s0 + u < n_slices ? t[u][e] : 0.f;
-        }
+        };
+        int s0 = 1;
+        if (CPT == 1)
+            for (; s0 + 4 < n_slices; s0 += 12) add_group(s0, std::integral_constant<int, 12>());
+        for (; s0 < n_slices; s0 += 4) add_group(s0, std::integral_constant<int, 4>());
 #pragma unroll
         for (int e = 0; e < 4; e++) {
             if (!ok) { a[j][e] = 0.f; v[j][e] = 0.f; }
