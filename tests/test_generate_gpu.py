@@ -159,6 +159,43 @@ def test_a_shrinking_batch_with_and_without_graphs(folders):
     assert runs[True, "sampled"] == runs[False, "sampled"] and [len(t) for t in runs[True, "sampled"]] == limits
 
 
+@pytest.mark.parametrize("temperature", [0.0, 0.8])
+def test_repetition_penalty_inside_the_graphs(folders, temperature):
+    """The penalty over the last 128 tokens, prompt included, when the recent tokens live in rings on the device that
+    the graphs extend themselves: the plain loop's tokens, with prompts shorter and longer than the window (a ring
+    that fills up, and one that is full from the start and overwrites its oldest place), through a batch that
+    shrinks into smaller graphs, and the same tokens as the loop that makes the choice on the host's side."""
+    from trapetum_amd import load_model
+    from trapetum_amd.sampling import initial_state
+    pcfg, pw = plain.read_folder(folders["B"])
+    lens, new = (120, 5, 140, 131, 64), 30
+    prompts = [random_tokens(n, pcfg["vocab_size"], 90 + i) for i, n in enumerate(lens)]
+    want = []
+    for i, p in enumerate(prompts):
+        state, seq, out = initial_state(11, i), list(p), []
+        for _ in range(new):
+            z = plain.repetition_penalty(plain.forward(pcfg, pw, seq)[-1], seq[-128:], 1.3)
+            if temperature > 0:
+                state = plain.xorshift64(state)
+                u = float(torch.tensor(plain.uniform_from_state(state), dtype=torch.float32))
+                tok = plain.sample(z, temperature, 0.9, 40, u)
+            else:
+                tok = int(z.argmax())
+            out.append(tok)
+            seq.append(tok)
+        want.append(out)
+    # tokens that end three of the requests at different steps, so that the batch shrinks
+    stops = {want[1][4], want[3][9], want[0][15]}
+    want_cut = [w[:min([w.index(t) for t in stops if t in w] + [new])] for w in want]
+    for use_graph in (True, False):
+        engine = load_model(folders["B"], dtype="float32", max_tokens_in_cache=4096, max_batch=8, use_graph=use_graph)
+        kw = dict(max_tokens=new, temperature=temperature, top_p=0.9, top_k=40, repetition_penalty=1.3, seed=11)
+        assert engine.generate(prompts, stop_ids=(), **kw) == want, use_graph
+        assert engine.generate(prompts, stop_ids=tuple(stops), **kw) == want_cut, use_graph
+        assert engine.cache.live_slots() == []
+    assert len(set(len(w) for w in want_cut)) > 2                 # the requests did end at different steps
+
+
 def test_graphs_are_dropped_beyond_their_number(folders):
     from .gpu_engine import load_gpu_model
     from trapetum_amd.engine.graphs import GraphedDecode

@@ -576,6 +576,16 @@ def test_sample_follows_the_plain_sampler(ops, vocab, temperature, top_k, top_p)
     assert got[2] == vocab - 1
 
 
+def test_recent_push(ops):
+    """A row's id goes to the place its cursor names, the cursor moves on and wraps at the ring's end."""
+    ring = torch.full((3, 5), -1, dtype=torch.int32, device=DEV)
+    cursor = torch.tensor([0, 4, 2], dtype=torch.int32, device=DEV)
+    ops.recent_push(torch.tensor([7, 8, 9], dtype=torch.int32, device=DEV), ring, cursor)
+    ops.recent_push(torch.tensor([1, 2, 3], dtype=torch.int32, device=DEV), ring, cursor)
+    assert ring.cpu().tolist() == [[7, 1, -1, -1, -1], [2, -1, -1, -1, 8], [-1, -1, 9, 3, -1]]
+    assert cursor.cpu().tolist() == [2, 1, 4]
+
+
 @pytest.mark.parametrize("vocab,window", [(256, 8), (256000, 128)])
 def test_repetition_penalty(ops, vocab, window):
     """Each distinct recent token once: z / penalty if z > 0 else z * penalty (runtime/src/bin/serve.rs:1330-1340)."""

@@ -177,6 +177,24 @@ extern "C" int tp_repetition_penalty(float* logits, int B, int V, const int* rec
     return tp_check_launch("repetition_penalty");
 }
 
+// The recent tokens of a row as a ring on the device, so that a captured decode graph can keep them by itself: the
+// row's chosen id goes to the place its cursor names, and the cursor moves on (the oldest id is overwritten once
+// the ring is full; the penalty reads the ring as a set, so the order inside it does not matter).
+__global__ void recent_push_k(const int* __restrict__ tokens, int* __restrict__ recent, int* __restrict__ cursor, int B, int R) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= B) return;
+    int at = cursor[i];
+    at = at < 0 || at >= R ? 0 : at;
+    recent[(size_t)i * R + at] = tokens[i];
+    cursor[i] = at + 1 == R ? 0 : at + 1;
+}
+
+extern "C" int tp_recent_push(const int* tokens, int* recent, int* cursor, int B, int R, void* stream) {
+    TP_REQUIRE(tokens && recent && cursor && B > 0 && R > 0, "recent_push: empty shape B=%d R=%d", B, R);
+    recent_push_k<<<tp_cdiv(B, 64), 64, 0, (hipStream_t)stream>>>(tokens, recent, cursor, B, R);
+    return tp_check_launch("recent_push");
+}
+
 // ---- temperature sampling over the top_k largest logits with a top_p cut, as the reference's next_tok
 // (runtime/src/bin/serve.rs:41-72): candidates sorted by logit descending (ties: smaller id first),
 // p = exp((z - max) / T) / sum, the shortest prefix whose cumulative mass reaches top_p, then a walk with

@@ -18,6 +18,7 @@ import collections
 import dataclasses
 from typing import List
 
+import numpy as np
 import torch
 
 from ..cache.slots import CacheError
@@ -98,19 +99,31 @@ class GraphRows:
         self.graphs, self.model, self.cache, self.slots = graphs, model, cache, slots
         self.requests = requests
         self.choice = sampler.graph_choice()
+        self.penalty = isinstance(self.choice[-1], tuple)
         self.nb = graph_rows(len(slots))
         self.place = list(range(len(slots)))          # row -> place in the graph's rows
 
     def start(self, ids):
-        self.graphs.rows(self.nb).tokens[:len(self.slots)].copy_(ids)
+        rows, n = self.graphs.rows(self.nb), len(self.slots)
+        rows.tokens[:n].copy_(ids)
+        if self.penalty:
+            # the rings start as the host knows them (the prompts' last tokens) and take the first ids on the device
+            rings = [Sampler.ring_of(r) for r in self.requests]
+            rt = self.model.rt
+            rows.recent[:n].copy_(rt.upload_i32(np.asarray([ring for ring, _ in rings], dtype=np.int32).reshape(-1)).view(n, -1))
+            rows.cursor[:n].copy_(rt.upload_i32(np.asarray([at for _, at in rings], dtype=np.int32)))
+            rt.ops.recent_push(rows.tokens, rows.recent, rows.cursor)
 
     def step(self, rows):
         cache = self.cache
         nb = graph_rows(len(rows))
         if nb < self.nb:                              # the live rows move into a smaller graph
-            old = self.graphs.rows(self.nb).tokens
-            index = torch.tensor([self.place[r] for r in rows], dtype=torch.long, device=old.device)
-            self.graphs.rows(nb).tokens[:len(rows)].copy_(old[index])
+            old, new = self.graphs.rows(self.nb), self.graphs.rows(nb)
+            index = torch.tensor([self.place[r] for r in rows], dtype=torch.long, device=old.tokens.device)
+            new.tokens[:len(rows)].copy_(old.tokens[index])
+            if self.penalty:
+                new.recent[:len(rows)].copy_(old.recent[index])
+                new.cursor[:len(rows)].copy_(old.cursor[index])
             self.place = [None] * len(self.place)
             for at, r in enumerate(rows):
                 self.place[r] = at
@@ -152,7 +165,9 @@ class BatchRun:
         self.slots = []
         self.pending = None                           # (rows, wait): ids chosen on the device that the host has not read
         self.rows = None
-        self.graphs = graphs if graphs is not None and sampler.graph_choice() is not None else None
+        self.graphs = graphs
+        # the host reads a step's ids before it enqueues the next only where it makes the choice itself from them
+        self.in_turn = graphs is None and sampler.needs_the_last_token
         self.steps = 0
 
     @property
@@ -200,7 +215,7 @@ class BatchRun:
     def advance(self):
         """Returns what the settled step emitted: [(request index, token)]."""
         rows, wait = self.pending
-        if self.sampler.needs_the_last_token:
+        if self.in_turn:
             # the next choice looks at the tokens chosen so far: the host reads them before it goes on
             ids = wait()
             self.sampler.record([self.requests[r] for r in rows], [ids[r] for r in rows])

@@ -10,7 +10,8 @@ replay reads its tokens, so a generation loop needs neither a launch nor a copy 
 fewer sequences than the graph has rows fills the rest with rows that stand for no sequence: they read and write
 the cache's spare page and spare slot.  What changes from step to step (slots, positions, lengths, page tables,
 the sampler's uniform numbers) lives at fixed device addresses, shared by the graphs of one batch size, that are
-refilled by one copy before each replay; page tables have the cache's widest width.  No memset node is
+refilled by one copy before each replay; page tables have the cache's widest width.  The recent tokens that a
+repetition penalty looks at are a ring per row on the device, which the graph itself extends by the id it chose.  No memset node is
 recorded: buffers are filled by copies and kernels.  The least recently used graphs are dropped beyond
 `max_graphs`.
 """
@@ -19,6 +20,7 @@ import collections
 import numpy as np
 import torch
 
+from ..sampling.sampler import RECENT_WINDOW
 from .batch import StaticStep, StepContext, step_arrays
 
 
@@ -45,6 +47,8 @@ class _Rows:
         self.static = StaticStep(rt, cache, nb, extra=nb)
         self.tokens = torch.zeros(nb, dtype=torch.int32, device=rt.device)
         self.uniforms = self.static.extra_view().view(torch.float32)
+        self.recent = torch.full((nb, RECENT_WINDOW), -1, dtype=torch.int32, device=rt.device)     # rings of chosen and prompt ids
+        self.cursor = torch.zeros(nb, dtype=torch.int32, device=rt.device)                      # where a row's next id goes
 
 
 class _Captured:
@@ -69,14 +73,21 @@ class GraphedDecode:
         return self.rows_of[nb]
 
     def _choose(self, choice, logits, rows):
-        """choice: None, ("greedy",) or ("sample", temperature, top_k, top_p); the ids go where the tokens lie."""
+        """choice: None, ("greedy",) or ("sample", temperature, top_k, top_p), either followed by ("penalty", value):
+        then the logits of the rows' recent tokens are changed first.  The ids go where the tokens lie, and into the
+        rows' rings."""
         if choice is None:
             return
         ops = self.model.rt.ops
+        penalty = choice[-1][1] if isinstance(choice[-1], tuple) else None
+        if penalty is not None:
+            ops.apply_repetition_penalty(logits, rows.recent, penalty)
         if choice[0] == "greedy":
             ops.argmax(logits, out=rows.tokens)
         else:
             ops.sample(logits, choice[1], choice[2], choice[3], rows.uniforms, out=rows.tokens)
+        if penalty is not None:
+            ops.recent_push(rows.tokens, rows.recent, rows.cursor)
 
     def run(self, nb, slots, starts, choice=None, uniforms=None):
         """One decode step of `nb` rows (nb a size `graph_rows` gives): row i continues the sequence in slots[i], which

@@ -30,6 +30,7 @@ _CORE_SIGS = {
     "tp_argmax": [_P, _I, _I, _P, _P, _P],
     "tp_argmax_workspace_bytes": [_I, _I],
     "tp_repetition_penalty": [_P, _I, _I, _P, _I, _F, _P],
+    "tp_recent_push": [_P, _P, _P, _I, _I, _P],
     "tp_sample": [_P, _I, _I, _F, _I, _F, _P, _P, _P, _P],
     "tp_sample_workspace_bytes": [_I, _I],
     "tp_probe_stream": [_P, _L, _P, _I, _P],
@@ -503,6 +504,18 @@ class HipOps:
             raise KernelError("repetition_penalty: recent tokens must be contiguous int32 [rows, R]")
         self._call(self.lib, "tp_repetition_penalty", logits.data_ptr(), logits.shape[0], logits.shape[1],
                    recent.data_ptr(), recent.shape[1], float(penalty), self._stream())
+
+    def recent_push(self, tokens, recent, cursor):
+        """Row i's token goes into row i of the ring `recent` (int32 [rows, R]) at cursor[i], which moves on by one."""
+        self._dev(tokens, recent, cursor)
+        n = tokens.numel()
+        if tokens.dtype != torch.int32 or not tokens.is_contiguous() or cursor.dtype != torch.int32 or cursor.numel() != n \
+                or not cursor.is_contiguous():
+            raise KernelError("recent_push: tokens and cursors must be contiguous int32 of one length")
+        if recent.dtype != torch.int32 or recent.dim() != 2 or recent.shape[0] != n or not recent.is_contiguous():
+            raise KernelError("recent_push: the ring must be contiguous int32 [rows, R]")
+        self._call(self.lib, "tp_recent_push", tokens.data_ptr(), recent.data_ptr(), cursor.data_ptr(), n, recent.shape[1],
+                   self._stream())
 
     def sample(self, logits, temperature, top_k, top_p, uniforms, out=None):
         self._dev(logits, uniforms)

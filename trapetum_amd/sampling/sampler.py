@@ -77,17 +77,24 @@ class Sampler:
 
     @property
     def needs_the_last_token(self):
-        """Whether a choice depends on the tokens chosen before it (then the host must know them first)."""
+        """Whether a choice made on the host's side (`choose_on_device`) depends on the tokens chosen before it: then
+        the host must know them first.  (A captured graph keeps the recent tokens on the device instead.)"""
         return self.params.repetition_penalty > 1.0
 
     def graph_choice(self):
-        """The choice as a captured decode graph can make it by itself (see GraphedDecode.run), or None."""
+        """The choice as a captured decode graph makes it by itself (see GraphedDecode.run): ("greedy",) or
+        ("sample", temperature, top_k, top_p), followed by ("penalty", value) when the recent tokens count."""
         p = self.params
-        if self.needs_the_last_token:
-            return None
-        if p.temperature <= 0:
-            return ("greedy",)
-        return ("sample", float(p.temperature), int(p.top_k), float(p.top_p))
+        choice = ("greedy",) if p.temperature <= 0 else ("sample", float(p.temperature), int(p.top_k), float(p.top_p))
+        if p.repetition_penalty > 1.0:
+            choice += (("penalty", float(p.repetition_penalty)),)
+        return choice
+
+    @staticmethod
+    def ring_of(request):
+        """A request's recent tokens as a ring of RECENT_WINDOW places (-1: empty) and the place the next one takes."""
+        recent = list(request.recent)
+        return recent + [-1] * (RECENT_WINDOW - len(recent)), len(recent) % RECENT_WINDOW
 
     def choose(self, logits, requests):
         """logits fp32 [n, vocab] on the device (changed in place by a penalty); one RequestSampling per row.
