@@ -48,6 +48,9 @@ def test_bad_values():
     with pytest.raises(ConfigError, match="layer_types"):
         Gemma2Config.from_kwargs(**dict(TINY_A, layer_types=["full_attention"]))
     assert Gemma2Config.from_kwargs(**dict(TINY_A, attn_logit_softcapping=0.0)).attn_logit_softcapping is None
+    with pytest.raises(ConfigError, match="attention_bias"):          # read, and refused: never dropped in silence
+        Gemma2Config.from_kwargs(**dict(TINY_A, attention_bias=True))
+    assert Gemma2Config.from_kwargs(**dict(TINY_A, attention_bias=False)).attention_bias is False
     c = Gemma2Config.from_kwargs(**dict(TINY_A, layer_types=["full_attention", "sliding_attention"]))
     assert [c.layer_is_local(l) for l in range(2)] == [False, True]
 

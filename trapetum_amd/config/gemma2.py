@@ -38,6 +38,7 @@ class Gemma2Config(ModelConfig):
     bos_token_id: int = key("bos_token_id", "opt_int", None, doc="begin-of-sequence token")
     pad_token_id: int = key("pad_token_id", "opt_int", None, doc="padding token")
     layer_types: tuple = key("layer_types", "str_list", None, doc="per layer: sliding_attention or full_attention")
+    attention_bias: bool = key("attention_bias", "bool", False, doc="biases on the attention projections (Gemma-2 has none)")
 
     def validate(self):
         for name in ("hidden_size", "num_attention_heads", "num_key_value_heads",
@@ -62,6 +63,8 @@ class Gemma2Config(ModelConfig):
             v = getattr(self, name)
             if v is not None and v <= 0:          # the reference writes 0 for "off" (model/export_gemma.py:44-45)
                 setattr(self, name, None)
+        if self.attention_bias:               # no released Gemma-2 has them, and the reference's exporter reads none (model/export_gemma.py:53-61)
+            raise ConfigError("attention_bias is true: projections with a bias are not built (the products have no bias operand)")
         if self.layer_types is not None:
             if len(self.layer_types) != self.num_hidden_layers:
                 raise ConfigError(
@@ -80,4 +83,6 @@ class Gemma2Config(ModelConfig):
         d["model_type"] = "gemma2"
         if d.get("layer_types") is None:
             d.pop("layer_types", None)
+        if not d.get("attention_bias"):
+            d.pop("attention_bias", None)
         return d
