@@ -336,6 +336,9 @@ EXTEND_CASES = [
     (2, 2, 80, (33, 50), (0, 31), 16, 0, 0, 0.0),
     (16, 2, 128, (1300, 17, 129), (1234, 0, 128), 64, 512, 512, 30.0),
     (32, 1, 64, (90,), (89,), 16, 0, 0, 0.0),
+    # portions of hundreds of rows, which the rotation and cache write take 16 bytes at a time
+    (8, 4, 256, (700, 300), (300, 20), 64, 0, 0, 50.0),
+    (4, 2, 64, (600,), (200,), 16, 128, 128, 30.0),
 ]
 
 
