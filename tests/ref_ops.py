@@ -42,8 +42,10 @@ def add_rms_norm(stream, rows, gain_post, eps_post, gain_next, eps_next, out_dty
     return _norm(stream, gain_next, eps_next).to(out_dtype)
 
 
-def linear(x, w, out_dtype, softcap=None, defer=False):
+def linear(x, w, out_dtype, softcap=None, defer=False, bias=None):
     y = x.float() @ w.float().T
+    if bias is not None:
+        y = y + bias.float()
     if softcap:
         y = softcap * torch.tanh(y / softcap)
     return y.to(out_dtype)
@@ -61,13 +63,17 @@ def gated_linear(x, w_packed, inter, activation, out_dtype):
     return (act(g) * u)[:, :inter].to(out_dtype).contiguous()
 
 
-def _rotate(x, pos, inv_freq, rotary_dim):
+def _rotate(x, pos, inv_freq, rotary_dim, pairing="halves"):
     """x [M, heads, hd] fp32, pos [M]."""
     if inv_freq is None or rotary_dim == 0:
         return x
     half = rotary_dim // 2
     ang = pos.float()[:, None] * inv_freq[None, :]
     c, s = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+    if pairing == "neighbours":                          # pair d: elements 2d and 2d + 1
+        x0, x1 = x[..., 0:rotary_dim:2], x[..., 1:rotary_dim:2]
+        turned = torch.stack([x0 * c - x1 * s, x1 * c + x0 * s], dim=-1).reshape(*x.shape[:-1], rotary_dim)
+        return torch.cat([turned, x[..., rotary_dim:]], dim=-1)
     x0, x1 = x[..., :half], x[..., half:rotary_dim]
     return torch.cat([x0 * c - x1 * s, x1 * c + x0 * s, x[..., rotary_dim:]], dim=-1)
 
@@ -91,12 +97,12 @@ def gather_kv_prefix(table, k_pool, v_pool, rows_cap, cu_rows, keys):
 
 
 def rope_kv_write(q, k, v, H, KV, hd, inv_freq, rotary_dim, row_seq, row_pos, new_len, table,
-                  k_pool, v_pool, rows_cap, gathered=None):
+                  k_pool, v_pool, rows_cap, gathered=None, pairing="halves"):
     m = q.shape[0]
-    q.copy_(_rotate(q.float().reshape(m, H, hd), row_pos, inv_freq, rotary_dim).reshape(m, H * hd).to(q.dtype))
+    q.copy_(_rotate(q.float().reshape(m, H, hd), row_pos, inv_freq, rotary_dim, pairing).reshape(m, H * hd).to(q.dtype))
     if k is None:
         return
-    k.copy_(_rotate(k.float().reshape(m, KV, hd), row_pos, inv_freq, rotary_dim).reshape(m, KV * hd).to(k.dtype))
+    k.copy_(_rotate(k.float().reshape(m, KV, hd), row_pos, inv_freq, rotary_dim, pairing).reshape(m, KV * hd).to(k.dtype))
     page = k_pool.shape[2]
     for r in range(m):
         s, p = int(row_seq[r]), int(row_pos[r])

@@ -160,6 +160,22 @@ def test_linear_bf16(ops, algo, m, n, k):
     assert rel_l2(got_c, 3.0 * torch.tanh(ref / 3.0)) < 1e-5
 
 
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("m,n,k", [(1, 16, 8), (8, 2304, 2048), (70, 331, 88), (300, 77, 136)])
+def test_linear_with_a_bias(ops, dt, m, n, k):
+    """x @ w^T + bias, the bias added by a kernel of its own after whichever product kernel the shape takes."""
+    x, w = randn(m, k, dtype=DT[dt], seed=17), randn(n, k, dtype=DT[dt], seed=18, scale=0.05)
+    bias = randn(n, seed=19)
+    got = ops.linear(x, w, DT[dt], bias=bias)
+    ref = x.cpu().double() @ w.cpu().double().T + bias.cpu().double()
+    assert got.shape == (m, n) and rel_l2(got, ref) < (2e-6 if dt == "f32" else 4e-3)
+    assert rel_l2(ops.linear(x, w, DT[dt], defer=True, bias=bias), ref) < (2e-6 if dt == "f32" else 4e-3)   # never left in slices
+    with pytest.raises(Exception, match="bias"):
+        ops.linear(x, w, DT[dt], softcap=30.0, bias=bias)
+    with pytest.raises(Exception, match="bias"):
+        ops.linear(x, w, DT[dt], bias=bias[:-1].contiguous())
+
+
 @pytest.mark.parametrize("m,n,k", [(1, 16, 8), (3, 100, 71), (70, 331, 88), (5, 700, 2304)])
 def test_linear_f32(ops, m, n, k):
     x, w = randn(m, k, seed=9), randn(n, k, seed=10, scale=0.05)
@@ -269,6 +285,37 @@ def test_rope_kv_write(ops, dt, H, KV, hd, lens, page, rows_cap):
     assert torch.equal(pools[1].cpu(), pools_ref[1])
     # rows that no sequence owns stay untouched
     assert torch.equal((pools[0].cpu() != 0).any(dim=-1), (pools_ref[0] != 0).any(dim=-1))
+
+
+@pytest.mark.parametrize("dt", ["f32", "bf16"])
+@pytest.mark.parametrize("H,KV,hd,lens,page,rows_cap,rot", [
+    (4, 2, 16, (5, 11, 17), 16, 0, 16), (2, 2, 80, (33, 50), 16, 32, 48), (8, 4, 256, (300, 77), 64, 128, 256),
+    (3, 1, 64, (290,), 16, 0, 32)])
+def test_rope_kv_write_turning_neighbours(ops, dt, H, KV, hd, lens, page, rows_cap, rot):
+    """The other pairing: elements 2d and 2d + 1 turn together by the angle of pair d; few rows and many, a rotation over
+    part of the head, a ring."""
+    c = build_cache_case(DT[dt], H, KV, hd, lens, page, rows_cap, 24, 21)
+    inv_freq = (1.0 / (10000.0 ** (torch.arange(0, rot, 2, dtype=torch.float32) / rot)))
+    pools_ref = [torch.zeros(24, KV, page, hd, dtype=DT[dt]) for _ in range(2)]
+    pools = [p.to(DEV) for p in pools_ref]
+    q_ref, k_ref = c["q"].cpu().clone(), c["k"].cpu().clone()
+    halves = c["q"].cpu().clone()
+    ref_ops.rope_kv_write(q_ref, k_ref, c["v"].cpu(), H, KV, hd, inv_freq, rot, c["row_seq"], c["row_pos"],
+                          c["new_len"], c["table"], pools_ref[0], pools_ref[1], rows_cap, pairing="neighbours")
+    ref_ops.rope_kv_write(halves, None, None, H, KV, hd, inv_freq, rot, c["row_seq"], c["row_pos"], c["new_len"], c["table"],
+                          None, None, rows_cap)
+    assert rel_l2(halves, q_ref) > 0.1                       # the two pairings are not the same rotation
+    ops.rope_kv_write(c["q"], c["k"], c["v"], H, KV, hd, inv_freq.to(DEV), rot, c["row_seq"].to(DEV),
+                      c["row_pos"].to(DEV), c["new_len"].to(DEV), c["table"].to(DEV), pools[0], pools[1], rows_cap,
+                      pairing="neighbours")
+    t = 3e-6 if dt == "f32" else 6e-3
+    assert rel_l2(c["q"], q_ref) < t and rel_l2(c["k"], k_ref) < t
+    assert rel_l2(pools[0], pools_ref[0]) < t
+    assert torch.equal(pools[1].cpu(), pools_ref[1])
+    with pytest.raises(Exception, match="pairing"):
+        ops.rope_kv_write(c["q"], c["k"], c["v"], H, KV, hd, inv_freq.to(DEV), rot, c["row_seq"].to(DEV),
+                          c["row_pos"].to(DEV), c["new_len"].to(DEV), c["table"].to(DEV), pools[0], pools[1], rows_cap,
+                          pairing="thirds")
 
 
 ATTN_CASES = [

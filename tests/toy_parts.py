@@ -22,7 +22,8 @@ class EmaMixer(Mixer):
         self.decay = float(decay)
 
     def tensor_specs(self):
-        return {"proj.weight": TensorSpec((self.hidden_size, self.hidden_size))}
+        return {"proj.weight": TensorSpec((self.hidden_size, self.hidden_size)),
+                "proj.bias": TensorSpec((self.hidden_size,), init="norm")}
 
     def cache_spec(self):
         return StateSpec((self.hidden_size,), "float32")
@@ -30,6 +31,7 @@ class EmaMixer(Mixer):
     def bind(self, tensors, rt):
         self.rt = rt
         self.w = rt.matrix(tensors["proj.weight"])
+        self.b = tensors["proj.bias"].float().contiguous()
 
     def forward(self, ctx, x, site):
         state = site.state                                   # [slots, hidden] fp32, zero for a fresh slot
@@ -42,7 +44,7 @@ class EmaMixer(Mixer):
                 out[r] = s
             state[slot] = s
             row += count
-        return ctx.ops.linear(out.to(ctx.dtype), self.w, ctx.dtype)
+        return ctx.ops.linear(out.to(ctx.dtype), self.w, ctx.dtype, bias=self.b)       # a projection with a bias
 
 
 class SoftRoutedMLP(FeedForward):
@@ -98,7 +100,9 @@ class CenteredNorm(Norm):
 
 
 class SquaredPosition(Position):
-    """Rotary frequencies d -> 1 / (1 + d)^2 over part of the head: another table through the same interface."""
+    """Rotary frequencies d -> 1 / (1 + d)^2 over part of the head, turning neighbours (2d, 2d + 1) together: another
+    table and the other pairing through the same interface."""
+    pairing = "neighbours"
 
     def __init__(self, rotary_dim):
         self.rotary_dim = rotary_dim
@@ -183,7 +187,7 @@ def toy_reference(cfg, W, tokens):
         for r in range(T):
             s = cfg["decay"] * s + (1 - cfg["decay"]) * t[r]
             out.append(s)
-        return torch.stack(out) @ W[p + "mix.proj.weight"].T
+        return torch.stack(out) @ W[p + "mix.proj.weight"].T + W[p + "mix.proj.bias"]
 
     def attn(t, p, kv=None):
         H, hd, rot = cfg["heads"], cfg["head_size"], cfg["rotary"]
@@ -191,10 +195,11 @@ def toy_reference(cfg, W, tokens):
         ang = torch.arange(T, dtype=D)[:, None] * inv[None]
         c, s = torch.cos(ang)[:, None], torch.sin(ang)[:, None]
 
-        def rope(u):
+        def rope(u):                                       # neighbours turn together: pair d is elements 2d and 2d + 1
             u = u.reshape(T, H, hd)
-            a, b = u[..., :rot // 2], u[..., rot // 2:rot]
-            return torch.cat([a * c - b * s, b * c + a * s, u[..., rot:]], -1)
+            a, b = u[..., 0:rot:2], u[..., 1:rot:2]
+            turned = torch.stack([a * c - b * s, b * c + a * s], -1).reshape(T, H, rot)
+            return torch.cat([turned, u[..., rot:]], -1)
         q = rope(t @ W[p + "mix.q_proj.weight"].T)
         if kv is None:
             kv = (rope(t @ W[p + "mix.k_proj.weight"].T), (t @ W[p + "mix.v_proj.weight"].T).reshape(T, H, hd))

@@ -77,6 +77,9 @@ __device__ __forceinline__ float gelu_tanh_fast(float g) {
 // c1 = -2 * 0.7978845608 * log2(e), c3 = c1 * 0.044715, and SiLU, g / (1 + e^-g), with c1 = -log2(e), c3 = 0.  The
 // bf16 products' epilogues take the two constants (`epi.x`, `epi.y`) and have no branch on the activation's kind.
 enum { TP_ACT_GELU_TANH = 0, TP_ACT_SILU = 1 };
+// which elements of a head a rotation pairs: (f, f + rotary_dim / 2) as the reference does
+// (runtime/cuda/codebook_gemv.cu:219-230), or neighbours (2f, 2f + 1)
+enum { TP_ROPE_HALVES = 0, TP_ROPE_NEIGHBOURS = 1 };
 static inline bool tp_gate_constants(int act, float* c1, float* c3) {
     constexpr float LOG2E = 1.4426950408889634f;
     if (act == TP_ACT_GELU_TANH) { *c1 = -2.f * 0.7978845608f * LOG2E; *c3 = *c1 * 0.044715f; return true; }

@@ -381,7 +381,7 @@ rope_kv_write_k(T* __restrict__ q, long q_stride, T* __restrict__ k, long k_stri
                 const int* __restrict__ row_seq, const int* __restrict__ row_pos,
                 const int* __restrict__ new_len, const int* __restrict__ table, int table_w,
                 T* __restrict__ k_pool, T* __restrict__ v_pool, int page, int rows_cap, int hpb,
-                T* __restrict__ gk, T* __restrict__ gv, long g_stride, const int* __restrict__ key_row0) {
+                T* __restrict__ gk, T* __restrict__ gv, long g_stride, const int* __restrict__ key_row0, int pairing) {
     const int r = blockIdx.x;
     const int j_begin = blockIdx.y * hpb, j_end = min(j_begin + hpb, H + (k ? KV : 0));
     const int pos = row_pos[r];
@@ -402,31 +402,32 @@ rope_kv_write_k(T* __restrict__ q, long q_stride, T* __restrict__ k, long k_stri
         if (cached) cache_at = ((size_t)pg * KV * page + row % page) * hd;      // + kv head * page * hd
         if (gk) gather_at = (size_t)(key_row0[seq] + pos) * g_stride;           // + kv head * hd
     }
-    for (int f = threadIdx.x; f < half; f += blockDim.x) {     // one thread per pair (f, f + half)
+    for (int f = threadIdx.x; f < half; f += blockDim.x) {     // one thread per pair: elements (f, f + half), or neighbours (2f, 2f + 1)
         const float ang = (float)pos * inv_freq[f];
         const float c = cosf(ang), sn = sinf(ang);
+        const int e0 = pairing == TP_ROPE_NEIGHBOURS ? 2 * f : f, e1 = pairing == TP_ROPE_NEIGHBOURS ? 2 * f + 1 : f + half;
         for (int j = j_begin; j < j_end; j++) {
             const bool is_q = j < H;
             T* x = is_q ? q + (size_t)r * q_stride + (size_t)j * hd : k + (size_t)r * k_stride + (size_t)(j - H) * hd;
-            const float x0 = ld_f32(x + f), x1 = ld_f32(x + f + half);
+            const float x0 = ld_f32(x + e0), x1 = ld_f32(x + e1);
             const float y0 = x0 * c - x1 * sn, y1 = x1 * c + x0 * sn;
-            st_f32(x + f, y0);
-            st_f32(x + f + half, y1);
+            st_f32(x + e0, y0);
+            st_f32(x + e1, y1);
             if (is_q) continue;
             const T* vsrc = v + (size_t)r * v_stride + (size_t)(j - H) * hd;
             if (cached) {
                 const size_t off = cache_at + (size_t)(j - H) * page * hd;
-                st_f32(k_pool + off + f, y0);
-                st_f32(k_pool + off + f + half, y1);
-                v_pool[off + f] = vsrc[f];
-                v_pool[off + f + half] = vsrc[f + half];
+                st_f32(k_pool + off + e0, y0);
+                st_f32(k_pool + off + e1, y1);
+                v_pool[off + e0] = vsrc[e0];
+                v_pool[off + e1] = vsrc[e1];
             }
             if (gk) {
                 const size_t off = gather_at + (size_t)(j - H) * hd;
-                st_f32(gk + off + f, y0);
-                st_f32(gk + off + f + half, y1);
-                gv[off + f] = vsrc[f];
-                gv[off + f + half] = vsrc[f + half];
+                st_f32(gk + off + e0, y0);
+                st_f32(gk + off + e1, y1);
+                gv[off + e0] = vsrc[e0];
+                gv[off + e1] = vsrc[e1];
             }
         }
     }
@@ -536,10 +537,12 @@ extern "C" int tp_rope_kv_write(void* q, long q_stride, void* k, long k_stride, 
                                 const int* row_seq, const int* row_pos, const int* new_len,
                                 const int* table, int table_w, void* k_pool, void* v_pool,
                                 int page, int rows_cap, void* gk, void* gv, long g_stride, const int* key_row0,
-                                void* stream) {
+                                int pairing, void* stream) {
     TP_REQUIRE(M > 0 && H > 0 && hd > 0, "rope_kv_write: empty shape M=%d H=%d hd=%d", M, H, hd);
     TP_REQUIRE(rot >= 0 && rot <= hd && rot % 2 == 0, "rope_kv_write: rotary_dim %d must be even and at most head_dim %d", rot, hd);
     TP_REQUIRE(rot == 0 || inv_freq, "rope_kv_write: a rotation needs its frequency table");
+    TP_REQUIRE(pairing == TP_ROPE_HALVES || pairing == TP_ROPE_NEIGHBOURS, "rope_kv_write: pairing %d is neither halves (%d) nor neighbours (%d)",
+               pairing, TP_ROPE_HALVES, TP_ROPE_NEIGHBOURS);
     TP_REQUIRE(!k || (v && k_pool && v_pool && table && KV > 0 && page > 0 && table_w > 0),
                "rope_kv_write: keys without values, cache pools or page table");
     TP_REQUIRE(rows_cap >= 0 && (rows_cap == 0 || rows_cap % page == 0), "rope_kv_write: ring of %d rows is no multiple of the page size %d", rows_cap, page);
@@ -548,7 +551,7 @@ extern "C" int tp_rope_kv_write(void* q, long q_stride, void* k, long k_stride, 
     TP_REQUIRE(H + KV <= 65535, "rope_kv_write: %d heads exceed one launch", H + KV);
     const int heads = H + (k ? KV : 0);
     auto piecewise = [](const void* p, long stride) { return !p || ((uintptr_t)p % 16 == 0 && stride % 8 == 0); };
-    if (dtype == TP_BF16 && M >= 256 && hd % 8 == 0 && rot % 16 == 0 && rot <= 256 && piecewise(q, q_stride) && piecewise(k, k_stride) &&
+    if (pairing == TP_ROPE_HALVES && dtype == TP_BF16 && M >= 256 && hd % 8 == 0 && rot % 16 == 0 && rot <= 256 && piecewise(q, q_stride) && piecewise(k, k_stride) &&
         piecewise(v, v_stride) && piecewise(k_pool, 8) && piecewise(v_pool, 8) && piecewise(gk, g_stride) && piecewise(gv, g_stride)) {
         rope_kv_write_vec_k<<<M, 256, 0, s>>>((bf16_t*)q, q_stride, (bf16_t*)k, k_stride, (const bf16_t*)v, v_stride, H, KV, hd,
             inv_freq, rot, row_seq, row_pos, new_len, table, table_w, (bf16_t*)k_pool, (bf16_t*)v_pool, page, rows_cap,
@@ -562,11 +565,11 @@ extern "C" int tp_rope_kv_write(void* q, long q_stride, void* k, long k_stride, 
     if (dtype == TP_BF16)
         rope_kv_write_k<bf16_t><<<grid, threads, 0, s>>>((bf16_t*)q, q_stride, (bf16_t*)k, k_stride, (const bf16_t*)v, v_stride, H, KV, hd,
             inv_freq, rot, row_seq, row_pos, new_len, table, table_w, (bf16_t*)k_pool, (bf16_t*)v_pool, page, rows_cap, hpb,
-            (bf16_t*)gk, (bf16_t*)gv, g_stride, key_row0);
+            (bf16_t*)gk, (bf16_t*)gv, g_stride, key_row0, pairing);
     else if (dtype == TP_F32)
         rope_kv_write_k<float><<<grid, threads, 0, s>>>((float*)q, q_stride, (float*)k, k_stride, (const float*)v, v_stride, H, KV, hd,
             inv_freq, rot, row_seq, row_pos, new_len, table, table_w, (float*)k_pool, (float*)v_pool, page, rows_cap, hpb,
-            (float*)gk, (float*)gv, g_stride, key_row0);
+            (float*)gk, (float*)gv, g_stride, key_row0, pairing);
     else return tp_fail("rope_kv_write: unknown dtype %d", dtype);
     return tp_check_launch("rope_kv_write");
 }
@@ -622,6 +625,25 @@ extern "C" int tp_gather_kv_prefix(const void* k_pool, const void* v_pool, int d
 // ---- gated activation on a packed gate/up product: y [M, 2*Ip] fp32 with 16 gate columns, then the 16 up
 // columns of the same units, alternating.  out[m, i] = act(g) * u, act being gelu-tanh (runtime/cuda/codebook_gemv.cu:
 // 531-537) or SiLU (the reference's other feed-forward: runtime/cuda/codebook_gemv.cu:205-209), in float32 arithmetic.
+// ---- rows += bias: for products with a bias (the products themselves have no bias operand) ------------------------
+template <typename T>
+__global__ void add_bias_k(T* __restrict__ rows, const float* __restrict__ bias, long total, int N) {
+    for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x)
+        st_f32(rows + i, ld_f32(rows + i) + bias[i % N]);
+}
+
+extern "C" int tp_add_bias(void* rows, int dtype, const float* bias, int M, int N, void* stream) {
+    TP_REQUIRE(rows && bias && M > 0 && N > 0, "add_bias: empty shape M=%d N=%d", M, N);
+    const long total = (long)M * N;
+    long blocks = (total + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == TP_BF16) add_bias_k<bf16_t><<<(unsigned)blocks, 256, 0, s>>>((bf16_t*)rows, bias, total, N);
+    else if (dtype == TP_F32) add_bias_k<float><<<(unsigned)blocks, 256, 0, s>>>((float*)rows, bias, total, N);
+    else return tp_fail("add_bias: unknown dtype %d", dtype);
+    return tp_check_launch("add_bias");
+}
+
 template <typename T>
 __global__ void gated_act_k(const float* __restrict__ y, T* __restrict__ out, int I, int Ip2, int act) {
     const float* yr = y + (size_t)blockIdx.x * Ip2;

@@ -20,7 +20,7 @@ _CORE_SIGS = {
     "tp_gather_rows": [_P, _P, _P, _I, _I, _I, _P],
     "tp_sum_slices": [_P, _I, _L, _P, _I, _L, _P],
     "tp_rope_kv_write": [_P, _L, _P, _L, _P, _L, _I, _I, _I, _I, _I, _P, _I, _P, _P, _P, _P, _I, _P, _P, _I, _I,
-                         _P, _P, _L, _P, _P],
+                         _P, _P, _L, _P, _I, _P],
     "tp_gather_kv_prefix": [_P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P, _P, _P, _I, _P, _P, _L, _P],
     "tp_gated_act": [_P, _P, _I, _I, _I, _I, _P],
     "tp_linear": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P, _L, _I, _I, _P],
@@ -31,6 +31,7 @@ _CORE_SIGS = {
     "tp_argmax_workspace_bytes": [_I, _I],
     "tp_repetition_penalty": [_P, _I, _I, _P, _I, _F, _P],
     "tp_recent_push": [_P, _P, _P, _I, _I, _P],
+    "tp_add_bias": [_P, _I, _P, _I, _I, _P],
     "tp_sample": [_P, _I, _I, _F, _I, _F, _P, _P, _P, _P],
     "tp_sample_workspace_bytes": [_I, _I],
     "tp_probe_stream": [_P, _L, _P, _I, _P],
@@ -45,6 +46,7 @@ _ATTN_SIGS = {
 }
 
 EPI_NONE, EPI_SOFTCAP, EPI_GATED = 0, 1, 2
+ROPE_PAIRINGS = {"halves": 0, "neighbours": 1}          # the kernel library's TP_ROPE_* enumerators
 GATE_ACTIVATIONS = {"gelu_tanh": 0, "silu": 1}       # what a gated product's epilogue can apply to the gate
 GATE_GROUP = 16
 
@@ -243,9 +245,12 @@ class HipOps:
         return out
 
     def rope_kv_write(self, q, k, v, H, KV, hd, inv_freq, rotary_dim, row_seq, row_pos, new_len, table,
-                      k_pool, v_pool, rows_cap, gathered=None):
+                      k_pool, v_pool, rows_cap, gathered=None, pairing="halves"):
         """Rotate q and k in place and write k, v into the cache.  gathered = (gk, gv, key_row0): the step's rows
-        also go into the buffers that `gather_kv_prefix` began, position t of sequence s into row key_row0[s] + t."""
+        also go into the buffers that `gather_kv_prefix` began, position t of sequence s into row key_row0[s] + t.
+        pairing: one of ROPE_PAIRINGS, which elements of a head turn together."""
+        if pairing not in ROPE_PAIRINGS:
+            raise KernelError(f"rope_kv_write: pairing '{pairing}' has no kernel ({', '.join(ROPE_PAIRINGS)})")
         self._dev(q, k, v, inv_freq, row_seq, row_pos, new_len, table, k_pool, v_pool)
         m = q.shape[0]
         qs = self._rows(q, "rope_kv_write q")
@@ -286,7 +291,7 @@ class HipOps:
                    new_len.data_ptr(), table.data_ptr() if k is not None else None, table_w,
                    k_pool.data_ptr() if k is not None else None, v_pool.data_ptr() if k is not None else None,
                    page, rows_cap, gk.data_ptr() if gk is not None else None, gv.data_ptr() if gv is not None else None,
-                   g_stride, row0.data_ptr() if row0 is not None else None, self._stream())
+                   g_stride, row0.data_ptr() if row0 is not None else None, ROPE_PAIRINGS[pairing], self._stream())
 
     def gather_kv_prefix(self, table, k_pool, v_pool, rows_cap, cu_rows, keys):
         """Buffers gk, gv [keys.total_keys, kv_heads * head_dim] with every sequence's cached positions
@@ -336,9 +341,19 @@ class HipOps:
                    self._stream())
         return out
 
-    def linear(self, x, w, out_dtype, softcap=None, defer=False):
-        """x @ w^T.  defer: the caller hands the result to `add_rms_norm` (or through `rows()`), so a product
-        computed in K slices may come back as SplitRows."""
+    def linear(self, x, w, out_dtype, softcap=None, defer=False, bias=None):
+        """x @ w^T (+ bias).  defer: the caller hands the result to `add_rms_norm` (or through `rows()`), so a product
+        computed in K slices may come back as SplitRows.  bias: float32 [rows of w], added by a kernel of its own
+        (the products have no bias operand), so a product with a bias is never left in slices."""
+        if bias is not None:
+            if softcap:
+                raise KernelError("linear: a bias and a cap together have no kernel")
+            y = self._linear(x, w, out_dtype, EPI_NONE, 0.0, 0)
+            self._dev(bias)
+            if bias.dtype != torch.float32 or bias.numel() != y.shape[1] or not bias.is_contiguous():
+                raise KernelError(f"linear: the bias must be contiguous float32 [{y.shape[1]}]")
+            self._call(self.lib, "tp_add_bias", y.data_ptr(), _code(y.dtype), bias.data_ptr(), y.shape[0], y.shape[1], self._stream())
+            return y
         if softcap:
             return self._linear(x, w, out_dtype, EPI_SOFTCAP, softcap, 0)
         return self._linear(x, w, out_dtype, EPI_NONE, 0.0, 0, defer=defer)

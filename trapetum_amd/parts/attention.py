@@ -64,7 +64,8 @@ class Attention(Mixer):
             raise ValueError(f"this attention sees {self.window or 'all'} keys back, the cache it reads keeps {site.spec.window}")
         table = ctx.page_table(site.group_index)
         rows_cap = site.rows_cap or 0
-        if ctx.mode == "decode" and ops.fuses_decode_step(ctx.dtype, H, KV, hd, site.k):
+        pairing = self.position.pairing
+        if ctx.mode == "decode" and pairing == "halves" and ops.fuses_decode_step(ctx.dtype, H, KV, hd, site.k):
             # one launch rotates, writes the cache and attends; the projections may stay in K slices until then
             qkv = ops.linear(x, self.w_qkv if owns_cache else self.w_qkv[:Q], ctx.dtype, defer=True)
             out = ops.attention_decode_step(qkv, H, KV, hd, self.inv_freq, self.position.rotary_dim, ctx.new_len,
@@ -86,7 +87,8 @@ class Attention(Mixer):
                 gk, gv = ops.gather_kv_prefix(table, site.k, site.v, rows_cap, ctx.cu_rows, keys)
                 gathered = (gk, gv, keys.key_row0_dev)
         ops.rope_kv_write(q, k, v, H, KV, hd, self.inv_freq, self.position.rotary_dim,
-                          ctx.row_seq, ctx.row_pos, ctx.new_len, table, site.k, site.v, rows_cap, gathered=gathered)
+                          ctx.row_seq, ctx.row_pos, ctx.new_len, table, site.k, site.v, rows_cap, gathered=gathered,
+                          pairing=pairing)
         if ctx.mode == "decode":
             out = ops.attention_decode(q, H, KV, hd, ctx.new_len, table, site.k, site.v, rows_cap,
                                        self.query_scale, self.softcap, self.window, ctx.dtype,

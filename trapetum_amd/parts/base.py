@@ -44,6 +44,7 @@ class Norm(Part):
 
 class Position(Part):
     rotary_dim = 0
+    pairing = "halves"        # which elements of a head a rotation turns together: "halves" (d, d + rotary_dim / 2) or "neighbours" (2d, 2d + 1)
 
     def inv_freq(self, device):
         raise NotImplementedError

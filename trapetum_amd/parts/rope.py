@@ -6,6 +6,9 @@ itself (pairs (d, d + rotary_dim/2), angle = position * inv_freq[d], fp32 cos/si
 runtime/cuda/codebook_gemv.cu:219-230) is applied by the mixer's kernel just before
 the cache write; a variant with other frequencies only needs another table, which is
 how the reference carries its scaled variants too (runtime/src/lib.rs:1071-1076).
+`pairing` says which elements turn together: "halves", the reference's (d, d + rotary_dim/2),
+or "neighbours" (2d, 2d + 1); the kernel that fuses a decode step's rotation with its
+attention knows the halves only, so another pairing takes the separate launches.
 """
 import torch
 
@@ -14,11 +17,14 @@ from .base import Position
 
 
 class RotaryPosition(Position):
-    def __init__(self, rotary_dim, theta):
+    def __init__(self, rotary_dim, theta, pairing="halves"):
         if rotary_dim % 2:
             raise ValueError(f"rotary_dim {rotary_dim} must be even")
+        if pairing not in ("halves", "neighbours"):
+            raise ValueError(f"pairing '{pairing}' is neither halves nor neighbours")
         self.rotary_dim = rotary_dim
         self.theta = float(theta)
+        self.pairing = pairing
         self._tables = {}
 
     def inv_freq(self, device):
