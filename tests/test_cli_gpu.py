@@ -93,3 +93,28 @@ def test_switches(tmp_path):
     assert p.returncode == 0, p.stderr[-2000:]
     assert "tp_attn_decode_fused" not in p.stderr and "tp_attn_simple_decode" in p.stderr
     assert p.stdout.strip() == ids
+
+
+def test_bench_line(tmp_path):
+    """The measurement's one JSON line with two layers of the 2B sizes: the keys its readers rely on, a flat `config` of at
+    most 20 keys, fewer layers named beside the full number; more than one GPU is refused in one line with exit code 2."""
+    p = subprocess.run([sys.executable, "bench.py", "--layers", "2", "--steps", "4", "--warmup", "2"], cwd=ROOT,
+                       capture_output=True, text=True, timeout=600)
+    assert p.returncode == 0, p.stderr[-2000:]
+    lines = [l for l in p.stdout.splitlines() if l.startswith("{")]
+    assert len(lines) == 1
+    d = json.loads(lines[0])
+    for k in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling",
+              "vs_baseline", "dtype", "data", "config", "prefill", "roofline", "points"):
+        assert k in d, k
+    assert d["n_gpus"] == 1 and d["steps"] == 4 and d["warmup"] == 2 and d["higher_is_better"] is True and d["dtype"] == "bf16"
+    assert d["value"] > 0 and abs(d["value"] - 8 * 1e3 / d["ms_per_step"]) < 0.01 * d["value"]
+    c = d["config"]
+    assert len(c) <= 20 and all(not isinstance(v, (dict, list)) for v in c.values())
+    assert c["layers"] == 2 and c["layers_full"] == 26 and c["global_batch"] == 8 and c["hidden"] == 2304
+    assert set(d["prefill"]) >= {"value", "tokens", "ms", "frac"} and d["prefill"]["tokens"] == 2048
+    r = d["roofline"]
+    assert r["bound"] == "hbm" and r["unit"] == "GB/s" and r["peak"] == 8000.0 and abs(r["frac"] - r["achieved"] / r["peak"]) < 1e-3
+    assert set(d["points"]) >= {"decode_b1", "decode_b64"}
+    p = subprocess.run([sys.executable, "bench.py", "--gpus", "2"], cwd=ROOT, capture_output=True, text=True, timeout=120)
+    assert p.returncode == 2 and len((p.stdout + p.stderr).strip().splitlines()) == 1
