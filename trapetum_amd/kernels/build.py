@@ -63,7 +63,7 @@ def _headers(sources):
 
 def _stamp(sources, defines):
     h = hashlib.sha256()
-    h.update(" ".join(FLAGS + defines).encode())
+    h.update(" ".join(FLAGS + list(defines)).encode())
     for name in list(sources) + _headers(sources):
         with open(os.path.join(CSRC, name), "rb") as f:
             h.update(name.encode())
