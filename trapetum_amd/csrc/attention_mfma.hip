@@ -12,6 +12,7 @@
 // ends up with 4 keys of ONE query, so the softmax statistics are per-lane scalars and the probabilities are
 // already laid out as the B operand of the second product.
 #include "common.h"
+#include <type_traits>
 #include "error_channel.h"
 
 #ifndef TP_HD
@@ -514,57 +515,79 @@ attn_decode_k(DecodeArgs a) {
     // p writes the key and the value into the cache before anyone in the block reads that row ---------------------
     if (a.qkv) {
         const int half = a.rot >> 1, rest = HD - a.rot;
-        auto val = [&](long col) -> float {
-            if (a.qkv_f32) {                     // slices added in order, four loads in flight at a time
-                const float* src = (const float*)a.qkv + (size_t)seq * a.row_stride + col;
-                float t = 0.f;
+        // NC columns of the sequence's row at once: their loads are asked for together (of float32 slices four slices
+        // at a time, added in slice order), so that a thread pays one trip to memory for all it needs, not one a column
+        auto vals = [&](auto ncol, const long* cols, float* out) {
+            constexpr int NC = decltype(ncol)::value;
+            if (a.qkv_f32) {
+                const float* src = (const float*)a.qkv + (size_t)seq * a.row_stride;
+#pragma unroll
+                for (int c = 0; c < NC; c++) out[c] = 0.f;
                 for (int s0 = 0; s0 < a.n_slices; s0 += 4) {
-                    float part[4];
+                    float part[NC][4];
 #pragma unroll
-                    for (int u = 0; u < 4; u++)
-                        part[u] = src[(size_t)(s0 + u < a.n_slices ? s0 + u : a.n_slices - 1) * a.slice_stride];
+                    for (int c = 0; c < NC; c++)
 #pragma unroll
-                    for (int u = 0; u < 4; u++) t += s0 + u < a.n_slices ? part[u] : 0.f;
+                        for (int u = 0; u < 4; u++)
+                            part[c][u] = src[(size_t)(s0 + u < a.n_slices ? s0 + u : a.n_slices - 1) * a.slice_stride + cols[c]];
+#pragma unroll
+                    for (int c = 0; c < NC; c++)
+#pragma unroll
+                        for (int u = 0; u < 4; u++) out[c] += s0 + u < a.n_slices ? part[c][u] : 0.f;
                 }
-                return t;
+            } else {
+                const bf16_t* src = (const bf16_t*)a.qkv + (size_t)seq * a.row_stride;
+#pragma unroll
+                for (int c = 0; c < NC; c++) out[c] = bf16_to_f32(src[cols[c]]);
             }
-            return bf16_to_f32(((const bf16_t*)a.qkv)[(size_t)seq * a.row_stride + col]);
         };
-        for (int idx = tid; idx < G * half; idx += DTH) {
-            const int qi = idx / half, f = idx - qi * half;
-            const long col = (long)(kvh * G + qi) * HD;
-            const float ang = (float)p * a.inv_freq[f];
-            const float cs = cosf(ang), sn = sinf(ang);
-            const float x0 = val(col + f), x1 = val(col + f + half);
-            q_lds[qi * HD + f] = f32_to_bf16(x0 * cs - x1 * sn);
-            q_lds[qi * HD + f + half] = f32_to_bf16(x1 * cs + x0 * sn);
-        }
-        for (int idx = tid; idx < G * rest; idx += DTH) {
-            const int qi = idx / rest, d = a.rot + idx - qi * rest;
-            q_lds[qi * HD + d] = f32_to_bf16(val((long)(kvh * G + qi) * HD + d));
-        }
-        if (a.write_kv && p < t_begin + chunk) {                  // t_begin <= p holds here: this slice has position p
+        // the slice that holds position p (t_begin <= p holds here) also rotates the new key and writes it and the value
+        // into the cache: thread f < rot/2 does that beside its pair of the first query head, whose angle is the same
+        const bool writer = a.write_kv && p < t_begin + chunk;
+        bf16_t* kdst = nullptr;
+        bf16_t* vdst = nullptr;
+        if (writer) {
             int row = a.rows_cap > 0 ? p % a.rows_cap : p;
             const int pg = table[row >> page_shift];
             const size_t at = (((size_t)pg * a.KV + kvh) * a.page + (row & page_mask)) * HD;
-            bf16_t* kdst = a.k_pool + at;
-            bf16_t* vdst = a.v_pool + at;
-            const long kcol = (long)(a.H + kvh) * HD, vcol = (long)(a.H + a.KV + kvh) * HD;
-            for (int f = tid; f < half; f += DTH) {
-                const float ang = (float)p * a.inv_freq[f];
-                const float cs = cosf(ang), sn = sinf(ang);
-                const float x0 = val(kcol + f), x1 = val(kcol + f + half);
-                kdst[f] = f32_to_bf16(x0 * cs - x1 * sn);
-                kdst[f + half] = f32_to_bf16(x1 * cs + x0 * sn);
-                vdst[f] = f32_to_bf16(val(vcol + f));
-                vdst[f + half] = f32_to_bf16(val(vcol + f + half));
-            }
-            for (int d = a.rot + tid; d < HD; d += DTH) {
-                kdst[d] = f32_to_bf16(val(kcol + d));
-                vdst[d] = f32_to_bf16(val(vcol + d));
-            }
-            __threadfence_block();
+            kdst = a.k_pool + at;
+            vdst = a.v_pool + at;
         }
+        const long kcol = (long)(a.H + kvh) * HD, vcol = (long)(a.H + a.KV + kvh) * HD;
+        for (int idx = tid; idx < G * half; idx += DTH) {
+            const int qi = idx / half, f = idx - qi * half;
+            const long col = (long)(kvh * G + qi) * HD;
+            const bool kv = writer && idx < half;                 // then qi == 0 and f == idx
+            const long cols[6] = {col + f, col + f + half, kcol + f, kcol + f + half, vcol + f, vcol + f + half};
+            float x[6];
+            if (writer) vals(std::integral_constant<int, 6>(), cols, x);     // (the whole block takes this branch or the other)
+            else vals(std::integral_constant<int, 2>(), cols, x);
+            const float ang = (float)p * a.inv_freq[f];
+            float cs, sn;
+            sincosf(ang, &sn, &cs);
+            q_lds[qi * HD + f] = f32_to_bf16(x[0] * cs - x[1] * sn);
+            q_lds[qi * HD + f + half] = f32_to_bf16(x[1] * cs + x[0] * sn);
+            if (kv) {
+                kdst[f] = f32_to_bf16(x[2] * cs - x[3] * sn);
+                kdst[f + half] = f32_to_bf16(x[3] * cs + x[2] * sn);
+                vdst[f] = f32_to_bf16(x[4]);
+                vdst[f + half] = f32_to_bf16(x[5]);
+            }
+        }
+        for (int idx = tid; idx < G * rest; idx += DTH) {         // elements outside the rotation
+            const int qi = idx / rest, d = a.rot + idx - qi * rest;
+            const bool kv = writer && idx < rest;                 // then qi == 0
+            const long cols[3] = {(long)(kvh * G + qi) * HD + d, kcol + d, vcol + d};
+            float x[3];
+            if (writer) vals(std::integral_constant<int, 3>(), cols, x);
+            else vals(std::integral_constant<int, 1>(), cols, x);
+            q_lds[qi * HD + d] = f32_to_bf16(x[0]);
+            if (kv) {
+                kdst[d] = f32_to_bf16(x[1]);
+                vdst[d] = f32_to_bf16(x[2]);
+            }
+        }
+        if (writer) __threadfence_block();
     } else {
         for (int idx = tid; idx < G * HD; idx += DTH)
             q_lds[idx] = a.q[(size_t)seq * a.q_stride + (size_t)kvh * G * HD + idx];
