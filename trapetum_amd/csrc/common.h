@@ -59,6 +59,17 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
     return t;
 }
 
+// The same where `red` has not been used by the block before (a call's own 16 floats): one barrier less.
+__device__ __forceinline__ float block_sum_once(float v, float* red) {
+    v = wave_sum(v);
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = (blockDim.x + 63) >> 6;
+    if (lane == 0) red[wave] = v;
+    __syncthreads();
+    float t = 0.f;
+    for (int i = 0; i < nw; i++) t += red[i];
+    return t;
+}
+
 // ---- device: functions of the model ---------------------------------------------------------------
 __device__ __forceinline__ float gelu_tanh_f(float g) {
     return 0.5f * g * (1.0f + tanhf(0.7978845608f * (g + 0.044715f * g * g * g)));

@@ -211,7 +211,7 @@ __global__ void __launch_bounds__(NTH)
 add_rms_norm_vec_k(float* __restrict__ stream, const TR* __restrict__ rows, int n_slices, long slice_stride,
                    const float* __restrict__ gain_post, float eps_post,
                    const float* __restrict__ gain_next, float eps_next, T* __restrict__ out, int D) {
-    __shared__ float red[16];
+    __shared__ float red[16], red_next[16];             // one for each of the two sums: no barrier between their uses
     float* sr = stream + (size_t)blockIdx.x * D;
     const TR* ar = rows + (size_t)blockIdx.x * D;
     float a[CPT][4], v[CPT][4], gp[CPT][4], gn[CPT][4];
@@ -255,7 +255,7 @@ add_rms_norm_vec_k(float* __restrict__ stream, const TR* __restrict__ rows, int 
         for (int j = 0; j < CPT; j++)
 #pragma unroll
             for (int e = 0; e < 4; e++) ss += a[j][e] * a[j][e];
-        ss = block_sum(ss, red);
+        ss = block_sum_once(ss, red);
         scale_a = rsqrtf(ss / (float)D + eps_post);
     }
     float ss2 = 0.f;
@@ -272,7 +272,7 @@ add_rms_norm_vec_k(float* __restrict__ stream, const TR* __restrict__ rows, int 
         if (i < D) st4(sr + i, v[j]);
     }
     if (!gain_next) return;
-    ss2 = block_sum(ss2, red);
+    ss2 = block_sum_once(ss2, red_next);
     const float scale_s = rsqrtf(ss2 / (float)D + eps_next);
     T* orow = out + (size_t)blockIdx.x * D;
 #pragma unroll
