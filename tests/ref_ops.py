@@ -78,38 +78,10 @@ def _rotate(x, pos, inv_freq, rotary_dim, pairing="halves"):
     return torch.cat([x0 * c - x1 * s, x1 * c + x0 * s, x[..., rotary_dim:]], dim=-1)
 
 
-def gather_kv_prefix(table, k_pool, v_pool, rows_cap, cu_rows, keys):
-    """Buffers [keys.total_keys, KV * hd]: every sequence's cached positions prefix_lo .. start - 1 out of the cache."""
-    _, KV, page, hd = k_pool.shape
-    gk = torch.zeros((keys.total_keys, KV * hd), dtype=k_pool.dtype, device=k_pool.device)
-    gv = torch.zeros_like(gk)
-    for s in range(table.shape[0]):
-        count = int(cu_rows[s + 1]) - int(cu_rows[s])
-        cached = int(keys.cu_keys[s + 1]) - int(keys.cu_keys[s]) - count
-        for j in range(cached):
-            t = int(keys.prefix_lo[s]) + j
-            row = t % rows_cap if rows_cap else t
-            pg = int(table[s, row // page])
-            assert pg >= 0
-            gk[int(keys.cu_keys[s]) + j] = k_pool[pg, :, row % page, :].reshape(-1)
-            gv[int(keys.cu_keys[s]) + j] = v_pool[pg, :, row % page, :].reshape(-1)
-    return gk, gv
-
-
-def rope_kv_write(q, k, v, H, KV, hd, inv_freq, rotary_dim, row_seq, row_pos, new_len, table,
-                  k_pool, v_pool, rows_cap, gathered=None, pairing="halves"):
-    m = q.shape[0]
-    q.copy_(_rotate(q.float().reshape(m, H, hd), row_pos, inv_freq, rotary_dim, pairing).reshape(m, H * hd).to(q.dtype))
-    if k is None:
-        return
-    k.copy_(_rotate(k.float().reshape(m, KV, hd), row_pos, inv_freq, rotary_dim, pairing).reshape(m, KV * hd).to(k.dtype))
-    page = k_pool.shape[2]
-    for r in range(m):
+def _cache_rows(k, v, row_seq, row_pos, new_len, table, k_pool, v_pool, rows_cap):
+    KV, page, hd = k_pool.shape[1], k_pool.shape[2], k_pool.shape[3]
+    for r in range(k.shape[0]):
         s, p = int(row_seq[r]), int(row_pos[r])
-        if gathered is not None:
-            gk, gv, row0 = gathered
-            gk[int(row0[s]) + p] = k[r]
-            gv[int(row0[s]) + p] = v[r]
         row = p
         if rows_cap:
             if p + rows_cap < int(new_len[s]):
@@ -119,6 +91,21 @@ def rope_kv_write(q, k, v, H, KV, hd, inv_freq, rotary_dim, row_seq, row_pos, ne
         assert pg >= 0
         k_pool[pg, :, row % page, :] = k[r].reshape(KV, hd)
         v_pool[pg, :, row % page, :] = v[r].reshape(KV, hd)
+
+
+def rope_kv_write(q, k, v, H, KV, hd, inv_freq, rotary_dim, row_seq, row_pos, new_len, table,
+                  k_pool, v_pool, rows_cap, pairing="halves", write=True):
+    m = q.shape[0]
+    q.copy_(_rotate(q.float().reshape(m, H, hd), row_pos, inv_freq, rotary_dim, pairing).reshape(m, H * hd).to(q.dtype))
+    if k is None:
+        return
+    k.copy_(_rotate(k.float().reshape(m, KV, hd), row_pos, inv_freq, rotary_dim, pairing).reshape(m, KV * hd).to(k.dtype))
+    if write:
+        _cache_rows(k, v, row_seq, row_pos, new_len, table, k_pool, v_pool, rows_cap)
+
+
+def kv_write(k, v, KV, hd, row_seq, row_pos, new_len, table, k_pool, v_pool, rows_cap):
+    _cache_rows(k, v, row_seq, row_pos, new_len, table, k_pool, v_pool, rows_cap)
 
 
 def _attend(qrow, keys, vals, scale, softcap):
@@ -131,22 +118,33 @@ def _attend(qrow, keys, vals, scale, softcap):
 
 
 def attention_prefill(q, k, v, H, KV, hd, cu_rows, max_count, scale, softcap, window, out_dtype, row_seq=None, row_pos=None,
-                      keys=None):
-    """keys None: k, v are the step's own rows and positions count from each sequence's first row.  Else k, v are the
-    gathered buffers: sequence i's position t in row keys.key_row0[i] + t, row_pos absolute."""
+                      cached=None, shape=0):
+    """k, v: the step's own rows.  cached None: every sequence starts at position 0.  Else cached = (new_len, table,
+    k_pool, v_pool, rows_cap): sequence i's first row stands at new_len[i] - its count, and the positions before it are
+    read from the cache as it is."""
     m = q.shape[0]
     out = torch.zeros((m, H * hd), dtype=torch.float32, device=q.device)
     qf, kf, vf = q.float().reshape(m, H, hd), k.float().reshape(-1, KV, hd), v.float().reshape(-1, KV, hd)
     g = H // KV
     for i in range(len(cu_rows) - 1):
         a, b = int(cu_rows[i]), int(cu_rows[i + 1])
+        start, keys, vals = 0, kf[a:b], vf[a:b]
+        if cached is not None:
+            new_len, table, k_pool, v_pool, rows_cap = cached
+            page = k_pool.shape[2]
+            start = int(new_len[i]) - (b - a)
+            first = max(0, start - (window - 1)) if window else 0       # the earliest position any query of the step sees
+            pos = torch.arange(first, start)
+            rows = pos % rows_cap if rows_cap else pos
+            pages = table[i].long()[rows // page]
+            assert (pages >= 0).all()
+            keys = torch.cat([torch.zeros(first, KV, hd), k_pool[pages, :, rows % page, :].float().cpu(), kf[a:b].cpu()]).to(q.device)
+            vals = torch.cat([torch.zeros(first, KV, hd), v_pool[pages, :, rows % page, :].float().cpu(), vf[a:b].cpu()]).to(q.device)
         for r in range(a, b):
-            p = r - a if keys is None else int(row_pos[r])
-            row0 = a if keys is None else int(keys.key_row0[i])
+            p = start + r - a
             lo = 0 if not window else max(0, p - window + 1)
             for h in range(H):
-                out[r, h * hd:(h + 1) * hd] = _attend(qf[r, h], kf[row0 + lo:row0 + p + 1, h // g],
-                                                      vf[row0 + lo:row0 + p + 1, h // g], scale, softcap)
+                out[r, h * hd:(h + 1) * hd] = _attend(qf[r, h], keys[lo:p + 1, h // g], vals[lo:p + 1, h // g], scale, softcap)
     return out.to(out_dtype)
 
 

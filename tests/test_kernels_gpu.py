@@ -331,10 +331,12 @@ ATTN_CASES = [
 ]
 
 
-@pytest.mark.parametrize("plain", [True, False])
+@pytest.mark.parametrize("kernel", ["plain", 0, 1, 2, 3])
 @pytest.mark.parametrize("dt", ["f32", "bf16"])
 @pytest.mark.parametrize("H,KV,hd,lens,page,window,rows_cap,cap", ATTN_CASES)
-def test_attention_prefill(ops, plain, dt, H, KV, hd, lens, page, window, rows_cap, cap):
+def test_attention_prefill(ops, kernel, dt, H, KV, hd, lens, page, window, rows_cap, cap):
+    """kernel: the plain one, or the matrix-core kernel with its block shape (0: its own choice)."""
+    plain = kernel == "plain"
     if dt == "f32" and not plain:
         pytest.skip("float32 runs on the plain kernel only")
     c = build_cache_case(DT[dt], H, KV, hd, lens, page, rows_cap, 24, 30)
@@ -344,17 +346,21 @@ def test_attention_prefill(ops, plain, dt, H, KV, hd, lens, page, window, rows_c
     ops.force_plain_attention = plain
     try:
         got = ops.attention_prefill(c["q"], c["k"], c["v"], H, KV, hd, c["cu"].to(DEV), max(lens), scale, cap, window,
-                                    DT[dt], row_seq=c["row_seq"].to(DEV), row_pos=c["row_pos"].to(DEV))
+                                    DT[dt], row_seq=c["row_seq"].to(DEV), row_pos=c["row_pos"].to(DEV),
+                                    shape=0 if plain else kernel)
     finally:
         ops.force_plain_attention = False
     assert rel_l2(got, ref) < (3e-6 if dt == "f32" else 8e-3)
 
 
+@pytest.mark.parametrize("shape", [0, 1, 2, 3])
 @pytest.mark.parametrize("H,KV,hd,lens,window,cap", [(64, 8, 16, (450, 130, 64), 100, 30.0), (8, 4, 256, (3300,), 0, 50.0),
-                                                    (8, 4, 256, (1000, 77), 300, 0.0)])
-def test_attention_prefill_many_tiles(ops, H, KV, hd, lens, window, cap):
-    """Steps of many and of few query tiles (the kernel cuts them into blocks of 64 and of 32 queries), against
-    dense masked attention per sequence and head."""
+                                                    (8, 4, 256, (1000, 77), 300, 0.0), (12, 4, 128, (700, 1), 0, 30.0),
+                                                    (6, 2, 80, (333,), 64, 0.0), (4, 4, 48, (97, 300), 0, 20.0)])
+def test_attention_prefill_many_tiles(ops, shape, H, KV, hd, lens, window, cap):
+    """Steps of many and of few query tiles in every block shape of the kernel (column groups that are heads of a kv
+    head or further positions; one, two or four groups of keys), against dense masked attention per sequence and
+    head."""
     m, g, scale = sum(lens), H // KV, 1.0 / math.sqrt(hd * 0.7)
     q, k, v = (randn(m, n * hd, dtype=torch.bfloat16, seed=40 + i) for i, n in enumerate((H, KV, KV)))
     cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
@@ -369,7 +375,7 @@ def test_attention_prefill_many_tiles(ops, H, KV, hd, lens, window, cap):
             if cap:
                 s = cap * torch.tanh(s / cap)
             ref[rows, h] = torch.softmax(s.masked_fill(hidden, float("-inf")), dim=-1) @ vs[:, h // g]
-    got = ops.attention_prefill(q, k, v, H, KV, hd, cu.to(DEV), max(lens), scale, cap, window, torch.bfloat16)
+    got = ops.attention_prefill(q, k, v, H, KV, hd, cu.to(DEV), max(lens), scale, cap, window, torch.bfloat16, shape=shape)
     assert rel_l2(got.reshape(m, H, hd), ref) < 8e-3
 
 
@@ -389,14 +395,15 @@ EXTEND_CASES = [
 ]
 
 
-@pytest.mark.parametrize("plain", [True, False])
+@pytest.mark.parametrize("kernel", ["plain", 0, 1, 2, 3])
 @pytest.mark.parametrize("dt", ["f32", "bf16"])
 @pytest.mark.parametrize("H,KV,hd,lens,starts,page,window,rows_cap,cap", EXTEND_CASES)
-def test_attention_over_cached_positions_and_the_steps_rows(ops, plain, dt, H, KV, hd, lens, starts, page, window, rows_cap, cap):
-    """A step that continues sequences by several tokens: the cached positions are copied out of the (ring) cache,
-    the step's rows are rotated, cached and added to them, and the queries attend over both.  Against whole-sequence
-    attention of the reference; afterwards the cache holds what a whole-sequence step would have left."""
-    from trapetum_amd.engine.batch import KeyGeometry
+def test_attention_over_cached_positions_and_the_steps_rows(ops, kernel, dt, H, KV, hd, lens, starts, page, window, rows_cap, cap):
+    """A step that continues sequences by several tokens: the queries attend over the cached positions, read in place
+    through the page table (a ring's rows too), and over the step's own rows, which are cached only afterwards.
+    Against whole-sequence attention of the reference; afterwards the cache holds what a whole-sequence step would
+    have left.  kernel: the plain one, or the matrix-core kernel with its block shape (0: its own choice)."""
+    plain = kernel == "plain"
     if dt == "f32" and not plain:
         pytest.skip("float32 runs on the plain kernel only")
     n_pages = 64
@@ -419,17 +426,18 @@ def test_attention_over_cached_positions_and_the_steps_rows(ops, plain, dt, H, K
     rows = torch.cat([torch.arange(int(c["cu"][i]) + s, int(c["cu"][i + 1])) for i, s in enumerate(starts)]).long()
     q, k, v = (c[name][rows.to(DEV)].contiguous() for name in ("q", "k", "v"))
     cu = torch.tensor([0] + list(torch.tensor(counts).cumsum(0)), dtype=torch.int32, device=DEV)
-    keys = KeyGeometry(starts, counts, window)
-    keys.cu_keys_dev, keys.key_row0_dev, keys.prefix_lo_dev = (torch.tensor(a, dtype=torch.int32, device=DEV)
-                                                                for a in (keys.cu_keys, keys.key_row0, keys.prefix_lo))
+    row_seq, row_pos, new_len, table = (c[name].to(DEV) for name in ("row_seq", "row_pos", "new_len", "table"))
+    row_seq, row_pos = row_seq[rows.to(DEV)].contiguous(), row_pos[rows.to(DEV)].contiguous()
     ops.force_plain_attention = plain
     try:
-        gk, gv = ops.gather_kv_prefix(c["table"].to(DEV), pools[0], pools[1], rows_cap, cu, keys)
-        ops.rope_kv_write(q, k, v, H, KV, hd, c["inv_freq"].to(DEV), hd, c["row_seq"][rows].to(DEV), c["row_pos"][rows].to(DEV),
-                          c["new_len"].to(DEV), c["table"].to(DEV), pools[0], pools[1], rows_cap,
-                          gathered=(gk, gv, keys.key_row0_dev))
-        got = ops.attention_prefill(q, gk, gv, H, KV, hd, cu, max(counts), scale, cap, window, DT[dt],
-                                    row_seq=c["row_seq"][rows].to(DEV), row_pos=c["row_pos"][rows].to(DEV), keys=keys)
+        ops.rope_kv_write(q, k, v, H, KV, hd, c["inv_freq"].to(DEV), hd, row_seq, row_pos, new_len, table, pools[0], pools[1],
+                          rows_cap, write=False)
+        before = [p.clone() for p in pools]
+        got = ops.attention_prefill(q, k, v, H, KV, hd, cu, max(counts), scale, cap, window, DT[dt],
+                                    row_seq=row_seq, row_pos=row_pos, cached=(new_len, table, pools[0], pools[1], rows_cap),
+                                    shape=0 if plain else kernel)
+        assert all(torch.equal(a, b) for a, b in zip(before, pools))       # neither the rotation nor the attention cached anything
+        ops.kv_write(k, v, KV, hd, row_seq, row_pos, new_len, table, pools[0], pools[1], rows_cap)
     finally:
         ops.force_plain_attention = False
     assert rel_l2(got, ref[rows]) < (3e-6 if dt == "f32" else 8e-3)

@@ -1,16 +1,15 @@
-// bf16 attention on the matrix cores for one head size (compiled with -DTP_HD=<head_dim>, a multiple of 16 up
-// to 256): a prefill kernel over a buffer of keys and values (the step's own rows, behind the cached positions
-// its queries still see when sequences continue) and a decode kernel over the paged cache.
+// bf16 attention of decode steps on the matrix cores for one head size (compiled with -DTP_HD=<head_dim>, a
+// multiple of 16 up to 256): one query per sequence and head over the paged cache.  (Steps of many queries:
+// attention_prefill.hip, in the same library.)
 //
 // Formula as the reference's attn_k (runtime/cuda/codebook_gemv.cu:240-270): score = (q . k) * scale, then
 // cap * tanh(score / cap) if a cap is set, softmax over the visible keys in fp32, weighted sum of v, query head
 // h reading kv head h / (heads / kv_heads).  The scale is an argument (rsqrt(head_dim) in the reference), and a
 // window W hides keys with p - t >= W (the reference has none: runtime/src/lib.rs:4455).
 //
-// Both kernels compute scores transposed, S^T = K . Q^T with v_mfma_f32_16x16x32_bf16: key rows are the A
-// operand (a lane holds 8 consecutive elements of one key: one 16-byte load), queries the B operand, and a lane
-// ends up with 4 keys of ONE query, so the softmax statistics are per-lane scalars and the probabilities are
-// already laid out as the B operand of the second product.
+// Scores are computed transposed, S^T = K . Q^T with v_mfma_f32_16x16x32_bf16: key rows are the A operand (a
+// lane holds 8 consecutive elements of one key: one 16-byte load), queries the B operand, and a lane ends up
+// with 4 keys of ONE query, so the softmax statistics are per-lane scalars.
 #include "common.h"
 #include <type_traits>
 #include "error_channel.h"
@@ -51,358 +50,6 @@ __device__ __forceinline__ bf16_t bf16_bits(float f) {
     return __builtin_bit_cast(bf16_t, b);
 }
 }  // namespace
-
-// =====================================================================================================
-// prefill: a sequence's keys and values are rows cu_keys[s] .. cu_keys[s + 1] - 1 of k and v, its queries the
-// rows cu_rows[s] .. of q, and the queries are the sequence's LAST positions: with Tk keys and Tq queries the
-// first query stands at key Tk - Tq (0 when every sequence starts in this step and the keys are its own rows;
-// more when cached positions were gathered in front of them).  Only differences of positions count.
-// Block = 64 or 32 queries of one (sequence, head); a wave owns 16 queries.  Key tiles of 32 go through LDS: K as
-// stored (row = key), V transposed (row = head element) with the keys of a tile permuted so that a lane's 8
-// probabilities meet the 8 values of the same keys in one 16-byte LDS read.
-// =====================================================================================================
-struct PrefillArgs {
-    const bf16_t* q; long q_stride; const bf16_t* k; long k_stride; const bf16_t* v; long v_stride;
-    int H, KV; const int* cu_rows; const int* cu_keys; float scale, cap; int window; bf16_t* out;
-    const bf16_t* vt; long vt_rows;      // V transposed: [kv head][head element][padded key slot], vt_rows slots per row
-};
-
-namespace {
-constexpr int BKV = 32;
-// LDS layouts of a key tile, both in rows of 128 bytes whose 16-byte chunks sit at chunk ^ (row & 7): the 16 rows
-// x 4 chunks that a fragment read touches then spread over the banks (padded rows lost 43 % of the LDS cycles to
-// conflicts).  K: sub-tiles of 64 head elements, a row per key.  V transposed: two head elements per row, 32 key
-// slots (64 bytes) each.
-constexpr int KSUB = (HDP + 63) / 64;
-__device__ __forceinline__ int k_at(int key, int d) {
-    return (d >> 6) * (BKV * 64) + key * 64 + ((((d & 63) >> 3) ^ (key & 7)) << 3) + (d & 7);
-}
-__device__ __forceinline__ int v_at(int d, int slot_chunk) {
-    return (d >> 1) * 64 + (((((d & 1) << 2) | slot_chunk) ^ ((d >> 1) & 7)) << 3);
-}
-}
-
-// V of the step, transposed once per layer so that the attention blocks copy it into LDS as it lies:
-// vt[kv head][d][slot], a sequence's keys in groups of 32 slots (its region padded to a multiple of 32), the keys
-// of a group permuted as the second product's operand wants them (key a*16 + g*4 + b at slot g*8 + a*4 + b).
-__device__ __forceinline__ int vt_base_of(const int* cu_rows, int seq) {
-    int base = 0;
-    for (int s = 0; s < seq; s++) base += (cu_rows[s + 1] - cu_rows[s] + BKV - 1) / BKV * BKV;
-    return base;
-}
-
-__global__ void __launch_bounds__(256)
-v_transpose_k(const bf16_t* __restrict__ v, long v_stride, int KV, const int* __restrict__ cu_rows,
-              bf16_t* __restrict__ vt, long vt_rows) {
-    __shared__ bf16_t tile[BKV][HD + 2];
-    const int seq = blockIdx.z, kvh = blockIdx.y, kt = blockIdx.x * BKV;
-    const int row0 = cu_rows[seq], T = cu_rows[seq + 1] - row0;
-    if (kt >= T) return;
-    const int base = vt_base_of(cu_rows, seq) + kt;
-    for (int i = threadIdx.x; i < BKV * NCH; i += 256) {
-        const int key = i / NCH, ch = i % NCH;
-        Frag f;
-        f.u = make_uint4(0, 0, 0, 0);
-        if (kt + key < T) f.u = *reinterpret_cast<const uint4*>(v + (size_t)(row0 + kt + key) * v_stride + (size_t)kvh * HD + ch * 8);
-#pragma unroll
-        for (int e = 0; e < 8; e++) tile[key][ch * 8 + e] = f.h[e];
-    }
-    __syncthreads();
-    for (int i = threadIdx.x; i < HD * BKV; i += 256) {          // consecutive threads: consecutive slots of one d
-        const int d = i / BKV, slot = i % BKV;
-        const int key = ((slot >> 2) & 1) * 16 + (slot >> 3) * 4 + (slot & 3);   // slot g*8 + a*4 + b holds key a*16 + g*4 + b
-        vt[((size_t)kvh * HD + d) * vt_rows + base + slot] = tile[key][d];
-    }
-}
-
-// Block = 8 waves in PGROUPS groups of PWAVES, PQ queries of one (sequence, head): wave w of every group owns
-// queries w*16 .. w*16+15.  Per round the block stages PGROUPS key tiles; group i takes the i-th, each group with its
-// own running softmax, so the chain of dependent rounds is 1/PGROUPS as long as the keys; at the end the other groups
-// hand (max, sum, unnormalised output) to group 0 through LDS.  A causal tile's work grows with its place in the
-// sequence, and a block occupies a CU alone: the late (long) tiles of every head carry the lowest block ids, so the
-// short ones fill in behind them, and a step of few tiles is cut into blocks of 32 queries instead of 64.
-namespace {
-constexpr int PTH = 512;                                         // threads of a prefill block
-constexpr int KS_ELEMS = KSUB * BKV * 64, VT_ELEMS = HD * BKV;    // one tile's K and V^T in LDS
-constexpr int MERGE_LANE = HD / 4 + 4;                           // a group's state per lane: its output tiles, max, sum (16-byte rows)
-template <int PQ> struct PrefillShape {                          // PQ: queries of a block
-    static constexpr int PWAVES = PQ / 16;                       // waves of a group
-    static constexpr int PGROUPS = PTH / 64 / PWAVES;
-    static constexpr int PKEYS = PGROUPS * BKV;                  // keys staged per round
-    static constexpr int MERGE_GROUP = PWAVES * 64 * MERGE_LANE;
-    static constexpr size_t TILE_BYTES = (size_t)PGROUPS * (KS_ELEMS + VT_ELEMS) * sizeof(bf16_t);
-    static constexpr size_t MERGE_BYTES = (size_t)(PGROUPS - 1) * MERGE_GROUP * sizeof(float);
-    static constexpr size_t LDS_BYTES = TILE_BYTES > MERGE_BYTES ? TILE_BYTES : MERGE_BYTES;
-    static_assert(LDS_BYTES <= 160 * 1024, "a round's tiles must fit the LDS of a CU");
-};
-}
-
-template <int PQ>
-__global__ void __launch_bounds__(PTH)
-attn_prefill_k(PrefillArgs a) {
-    using Shape = PrefillShape<PQ>;
-    constexpr int PWAVES = Shape::PWAVES, PGROUPS = Shape::PGROUPS, PKEYS = Shape::PKEYS, MERGE_GROUP = Shape::MERGE_GROUP;
-    extern __shared__ __attribute__((aligned(16))) unsigned char prefill_lds[];
-    bf16_t* Ks_all = reinterpret_cast<bf16_t*>(prefill_lds);                       // [group] tiles laid out by k_at
-    bf16_t* Vt_all = Ks_all + PGROUPS * KS_ELEMS;                                  // [group] tiles laid out by v_at
-    const int tid = threadIdx.x, grp = (tid >> 6) / PWAVES, wave = (tid >> 6) % PWAVES, lane = tid & 63, c = lane & 15, g = lane >> 4;
-    const bf16_t* Ks = Ks_all + grp * KS_ELEMS;
-    const bf16_t* Vt = Vt_all + grp * VT_ELEMS;
-    // late query tiles see the most keys: they are given the low block ids, which start first
-    const int seq = blockIdx.z, h = blockIdx.x % a.H, q0 = (gridDim.x / a.H - 1 - blockIdx.x / a.H) * PQ;
-    // rows of the queries (row0, Tq of them) and of the keys (krow0, T of them); query i stands at key qofs + i
-    const int row0 = a.cu_rows[seq], Tq = a.cu_rows[seq + 1] - row0;
-    if (q0 >= Tq) return;
-    const int krow0 = a.cu_keys[seq], T = a.cu_keys[seq + 1] - krow0, qofs = T - Tq;
-    const int kvh = h / (a.H / a.KV);
-    const int qw0 = qofs + q0 + wave * 16, qpos = qw0 + c;       // in key coordinates
-    const bool q_ok = qpos < T;
-
-    bf16x8 qf[KSTEPS];
-#pragma unroll
-    for (int ks = 0; ks < KSTEPS; ks++) {
-        const int d0 = ks * 32 + g * 8;
-        qf[ks] = ld_frag(a.q + (size_t)(row0 + (q_ok ? qpos - qofs : 0)) * a.q_stride + (size_t)h * HD + d0, q_ok && d0 < HD);
-    }
-    if (HDP > HD)                                   // the padding columns of K stay zero for the whole kernel
-        for (int i = tid; i < PKEYS * (HDP - HD); i += PTH) {
-            const int key = i / (HDP - HD);
-            Ks_all[(key / BKV) * KS_ELEMS + k_at(key % BKV, HD + i % (HDP - HD))] = 0;
-        }
-
-    f32x4 o[HD / 16];
-#pragma unroll
-    for (int dt = 0; dt < HD / 16; dt++) o[dt] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    float m_i = -INFINITY, l_i = 0.f;                                // the running maximum in units of log 2
-    constexpr float LOG2E = 1.4426950408889634f;
-    const float tanh_in = a.cap > 0.f ? 2.f * LOG2E * a.scale / a.cap : 0.f, cap2 = a.cap * LOG2E, scale2 = a.scale * LOG2E;
-    // the keys a lane's query sees: seen_lo .. seen_lo + seen_span
-    const int seen_lo = a.window > 0 ? max(0, qpos - a.window + 1) : 0;
-    const unsigned seen_span = (unsigned)max(0, min(qpos, T - 1) - seen_lo);
-
-    int k_lo = a.window > 0 ? max(0, qofs + q0 - a.window + 1) : 0;
-    k_lo &= ~(BKV - 1);
-    const int k_hi = min(T, qofs + q0 + PQ);
-    // a round's rows travel global memory -> registers (one round ahead, while the round before is being used) ->
-    // LDS; K as stored, V from its transposed copy: HD rows of PKEYS slots per round
-    constexpr int VCH = PKEYS / 8;                                  // 16-byte chunks of a head element's slots in a round
-    constexpr int KTASKS = (PKEYS * NCH + PTH - 1) / PTH;           // (key, 16-byte chunk) per thread
-    constexpr int VTASKS = (HD * VCH + PTH - 1) / PTH;              // (head element, chunk of its slots)
-    bf16x8 fk[KTASKS], fv[VTASKS];
-    // Addresses: a byte offset per thread from base pointers that are the same for the whole block and move with the
-    // round (scalar work).  A chunk the round does not need reads the round's first chunk instead, so that every load
-    // is issued without a branch and nothing is computed per round and lane but a comparison and a selection.
-    constexpr bool K_EVEN = PTH % NCH == 0;                         // then task t's key is task 0's + t * PTH / NCH
-    const char* const k_origin = reinterpret_cast<const char*>(a.k + (size_t)krow0 * a.k_stride + (size_t)kvh * HD);
-    const char* const v_origin = reinterpret_cast<const char*>(a.vt + (size_t)kvh * HD * a.vt_rows + vt_base_of(a.cu_keys, seq));
-    const size_t k_row_bytes = (size_t)a.k_stride * sizeof(bf16_t), v_row_bytes = (size_t)a.vt_rows * sizeof(bf16_t);
-    unsigned koff[K_EVEN ? 1 : KTASKS];
-    int kkey[K_EVEN ? 1 : KTASKS];
-#pragma unroll
-    for (int t = 0; t < (K_EVEN ? 1 : KTASKS); t++) {
-        const int i = tid + t * PTH, key = i / NCH, ch = i % NCH;
-        kkey[t] = i < PKEYS * NCH ? key : PKEYS;                    // PKEYS: no round needs it
-        koff[t] = (unsigned)(key * (int)k_row_bytes + ch * 16);
-    }
-    const int v_d = tid / VCH, v_part = tid % VCH, v_tile_key = (v_part >> 2) * BKV;     // task t: head element v_d + t * PTH / VCH
-    const unsigned voff = (unsigned)(v_d * (int)v_row_bytes + v_part * 16);
-    auto fetch = [&](int kt) {
-        const int left = min(k_hi - kt, PKEYS);                     // keys of the round that some query sees
-        const char* const kb = k_origin + (size_t)kt * k_row_bytes;
-        const char* const vb = v_origin + (size_t)kt * sizeof(bf16_t);
-#pragma unroll
-        for (int t = 0; t < KTASKS; t++) {
-            unsigned off;
-            if constexpr (K_EVEN) off = kkey[0] + t * (PTH / NCH) < left ? koff[0] + (unsigned)(t * (PTH / NCH)) * (unsigned)k_row_bytes : 0u;
-            else off = kkey[t] < left ? koff[t] : 0u;
-            fk[t] = *reinterpret_cast<const bf16x8*>(kb + off);
-        }
-#pragma unroll
-        for (int t = 0; t < VTASKS; t++) {
-            const bool need = v_d + t * (PTH / VCH) < HD && v_tile_key < left;      // a tile past the block's last key is never used
-            fv[t] = *reinterpret_cast<const bf16x8*>(vb + (need ? voff + (unsigned)(t * (PTH / VCH)) * (unsigned)v_row_bytes : 0u));
-        }
-    };
-    auto stage = [&]() {
-#pragma unroll
-        for (int t = 0; t < KTASKS; t++) {
-            const int i = tid + t * PTH;
-            const int key = i / NCH;
-            if (i < PKEYS * NCH)
-                *reinterpret_cast<bf16x8*>(Ks_all + (key / BKV) * KS_ELEMS + k_at(key % BKV, (i % NCH) * 8)) = fk[t];
-        }
-#pragma unroll
-        for (int t = 0; t < VTASKS; t++) {
-            const int i = tid + t * PTH;
-            const int d = i / VCH, part = i % VCH;                   // slots part*8 .. +7 of the round: tile part / 4
-            if (i < HD * VCH)
-                *reinterpret_cast<bf16x8*>(Vt_all + (part >> 2) * VT_ELEMS + v_at(d, part & 3)) = fv[t];
-        }
-    };
-    fetch(k_lo);
-    for (int kr = k_lo; kr < k_hi; kr += PKEYS) {
-        __syncthreads();                             // the round before has been used by every wave
-        stage();
-        __syncthreads();
-        if (kr + PKEYS < k_hi) fetch(kr + PKEYS);
-        const int kt = kr + grp * BKV;               // this group's tile
-        const bool visible = kt < k_hi && qw0 < T && kt <= qw0 + 15 && !(a.window > 0 && kt + BKV - 1 < qw0 - a.window + 1);
-        if (!visible) continue;                      // wave-uniform: every key of the tile is hidden from the wave's queries
-
-        f32x4 s[2];
-#pragma unroll
-        for (int j = 0; j < 2; j++) {
-            s[j] = (f32x4){0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int ks = 0; ks < KSTEPS; ks++) {
-                Frag kf;
-                kf.u = *reinterpret_cast<const uint4*>(Ks + k_at(j * 16 + c, ks * 32 + g * 8));
-                s[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qf[ks], s[j], 0, 0, 0);
-            }
-        }
-        // A lane holds the scores of keys kt + j*16 + g*4 + i for its query qpos.  From here on they are in units of
-        // log 2 (the constants carry the factor), so that every exponential is one instruction; the branches are the
-        // same for the whole wave.
-        float sc[8];
-        if (a.cap > 0.f) {                           // cap * tanh(x) = cap - 2 cap / (1 + e^(2x))
-#pragma unroll
-            for (int e = 0; e < 8; e++)
-                sc[e] = __builtin_fmaf(__builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(s[e >> 2][e & 3] * tanh_in)), -2.f * cap2, cap2);
-        } else {
-#pragma unroll
-            for (int e = 0; e < 8; e++) sc[e] = s[e >> 2][e & 3] * scale2;
-        }
-        // a tile every query of the wave sees whole needs no mask
-        const bool whole = kt + BKV - 1 <= qw0 && qw0 + 15 < T && (a.window <= 0 || qw0 + 15 - kt < a.window);
-        if (!whole) {
-            const int first = kt + g * 4 - seen_lo;
-#pragma unroll
-            for (int e = 0; e < 8; e++)
-                sc[e] = (unsigned)(first + (e >> 2) * 16 + (e & 3)) <= seen_span ? sc[e] : -INFINITY;
-        }
-        float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])), fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
-        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        const float m_new = fmaxf(m_i, mx);
-        const float m_ref = m_new == -INFINITY ? 0.f : m_new;      // a query that has seen no key yet: every term is 0
-        const float alpha = m_i == m_new ? 1.f : __builtin_amdgcn_exp2f(m_i - m_ref);
-        float sum = 0.f;
-        Frag pf;
-#pragma unroll
-        for (int e = 0; e < 8; e++) {
-            const float p = __builtin_amdgcn_exp2f(sc[e] - m_ref);
-            sum += p;
-            pf.h[e] = bf16_bits(p);
-        }
-        sum += __shfl_xor(sum, 16, 64);
-        sum += __shfl_xor(sum, 32, 64);
-        l_i = l_i * alpha + sum;
-        m_i = m_new;
-        if (__any(alpha != 1.f)) {                   // once the running maxima settle, nothing to rescale
-#pragma unroll
-            for (int dt = 0; dt < HD / 16; dt++) o[dt] = o[dt] * alpha;
-        }
-#pragma unroll
-        for (int dt = 0; dt < HD / 16; dt++) {
-            Frag vf;
-            vf.u = *reinterpret_cast<const uint4*>(Vt + v_at(dt * 16 + c, g));
-            o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf.v, o[dt], 0, 0, 0);
-        }
-    }
-    // ---- the other groups' states join group 0's, in the groups' order, all rescaled to the common maximum ---------
-    __syncthreads();                                 // the tiles in LDS are done with
-    float* merge = reinterpret_cast<float*>(prefill_lds) + (size_t)(wave * 64 + lane) * MERGE_LANE;
-    if (grp > 0) {
-        float* mine = merge + (size_t)(grp - 1) * MERGE_GROUP;
-#pragma unroll
-        for (int dt = 0; dt < HD / 16; dt++) *reinterpret_cast<f32x4*>(mine + dt * 4) = o[dt];
-        mine[HD / 4] = m_i;
-        mine[HD / 4 + 1] = l_i;
-    }
-    __syncthreads();
-    if (grp > 0 || !q_ok) return;
-    float m = m_i;
-#pragma unroll
-    for (int j = 0; j < PGROUPS - 1; j++) m = fmaxf(m, merge[(size_t)j * MERGE_GROUP + HD / 4]);
-    const float a0 = m_i == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m_i - m);
-    float l = l_i * a0;
-#pragma unroll
-    for (int dt = 0; dt < HD / 16; dt++) o[dt] = o[dt] * a0;
-#pragma unroll
-    for (int j = 0; j < PGROUPS - 1; j++) {
-        const float* theirs = merge + (size_t)j * MERGE_GROUP;
-        const float mj = theirs[HD / 4];
-        const float aj = mj == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mj - m);
-        l += theirs[HD / 4 + 1] * aj;
-#pragma unroll
-        for (int dt = 0; dt < HD / 16; dt++) o[dt] = o[dt] + *reinterpret_cast<const f32x4*>(theirs + dt * 4) * aj;
-    }
-    const float inv = 1.f / l;
-    bf16_t* orow = a.out + ((size_t)(row0 + qpos - qofs) * a.H + h) * HD;
-#pragma unroll
-    for (int dt = 0; dt < HD / 16; dt++) {
-        ushort4 pk;
-        pk.x = bf16_bits(o[dt][0] * inv); pk.y = bf16_bits(o[dt][1] * inv);
-        pk.z = bf16_bits(o[dt][2] * inv); pk.w = bf16_bits(o[dt][3] * inv);
-        *reinterpret_cast<ushort4*>(orow + dt * 16 + g * 4) = pk;
-    }
-}
-
-template <int PQ>
-static int prefill_launch(const PrefillArgs& a, int max_count, int H, int n_seq, hipStream_t stream) {
-    constexpr size_t lds = PrefillShape<PQ>::LDS_BYTES;
-    static bool configured = false;                                   // more LDS than a kernel gets without asking
-    if (!configured) {
-        hipError_t e = hipFuncSetAttribute((const void*)attn_prefill_k<PQ>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return tp_fail("attention prefill: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
-        configured = true;
-    }
-    attn_prefill_k<PQ><<<dim3(tp_cdiv(max_count, PQ) * H, 1, n_seq), PTH, lds, stream>>>(a);
-    return 0;
-}
-
-// elements of the transposed copy of V the prefill kernel needs as workspace (Mk: rows of keys)
-extern "C" long tp_attn_prefill_workspace_elems(int Mk, int KV, int n_seq) {
-    return (long)KV * HD * ((long)Mk + (long)BKV * n_seq + BKV);
-}
-
-// q: M rows of queries, sequence s's at cu_rows[s] ..; k, v: Mk rows of keys and values, sequence s's at
-// cu_keys[s] .. (null: the queries' own rows, cu_rows); a sequence's queries are its last positions.
-extern "C" int tp_attn_prefill(const void* q, long q_stride, const void* k, long k_stride, const void* v, long v_stride,
-                               int M, int H, int KV, const int* cu_rows, int n_seq, int max_count,
-                               const int* cu_keys, int Mk, int max_keys,
-                               float scale, float cap, int window, void* out, void* workspace, void* stream) {
-    TP_REQUIRE(M > 0 && H > 0 && KV > 0 && n_seq > 0 && max_count > 0, "attention prefill: empty shape");
-    TP_REQUIRE(H % KV == 0, "attention: %d query heads are no multiple of %d kv heads", H, KV);
-    if (!cu_keys) { cu_keys = cu_rows; Mk = M; max_keys = max_count; }
-    TP_REQUIRE(Mk >= M && max_keys >= max_count, "attention prefill: %d keys (at most %d a sequence) for %d queries (at most %d)", Mk, max_keys, M, max_count);
-    TP_REQUIRE(q_stride % 8 == 0 && k_stride % 8 == 0 && v_stride % 8 == 0 && (uintptr_t)q % 16 == 0 &&
-               (uintptr_t)k % 16 == 0 && (uintptr_t)v % 16 == 0, "attention prefill: rows must be 16-byte aligned");
-    TP_REQUIRE(n_seq <= 65535 && (long)tp_cdiv(max_count, 32) * H < (1L << 31), "attention prefill: %d heads / %d sequences exceed one launch", H, n_seq);
-    TP_REQUIRE(workspace && (uintptr_t)workspace % 16 == 0, "attention prefill: needs its 16-byte aligned workspace");
-    TP_REQUIRE(k_stride < (1L << 22) && (long)HD * ((long)Mk + (long)BKV * n_seq + BKV) < (1L << 30),
-               "attention prefill: %d rows of stride %ld exceed the kernel's 32-bit offsets", Mk, k_stride);
-    TP_REQUIRE(KV <= 65535, "attention prefill: %d kv heads exceed one launch", KV);
-    const long vt_rows = (long)Mk + (long)BKV * n_seq + BKV;        // every sequence's region is padded to whole groups
-    v_transpose_k<<<dim3(tp_cdiv(max_keys, BKV), KV, n_seq), 256, 0, (hipStream_t)stream>>>(
-        (const bf16_t*)v, v_stride, KV, cu_keys, (bf16_t*)workspace, vt_rows);
-    if (int rc = tp_check_launch("attention prefill (transpose of V)")) return rc;
-    PrefillArgs a{(const bf16_t*)q, q_stride, (const bf16_t*)k, k_stride, (const bf16_t*)v, v_stride, H, KV, cu_rows, cu_keys,
-                  scale, cap, window, (bf16_t*)out, (const bf16_t*)workspace, vt_rows};
-    // 64 queries a block stage each key once per 64 queries; 32 a block make twice the blocks, for grids that would
-    // not give every CU a block of 64 (measured, 8 heads of 256: 26 against 30 us at 512 tokens, 75 against 84 at
-    // 2,048, but 151 against 121 at 3,072; 32 heads of 128 at 2,048 tokens: 145 against 89 us)
-    static int cus = 0;
-    if (!cus) {
-        int dev = 0;
-        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
-            cus = 256;
-    }
-    const bool small = (long)tp_cdiv(max_count, 64) * H * n_seq <= cus;
-    if (int rc = small ? prefill_launch<32>(a, max_count, H, n_seq, (hipStream_t)stream)
-                       : prefill_launch<64>(a, max_count, H, n_seq, (hipStream_t)stream)) return rc;
-    return tp_check_launch("attention prefill");
-}
 
 // =====================================================================================================
 // decode: one query per sequence and head, keys and values in the paged cache.  A block owns one

@@ -11,10 +11,12 @@
 
 struct AttnSimpleArgs {
     const void* q; long q_stride;
-    // keys and values of the step itself (prefill): rows of sequence s start at cu_rows[s]
+    // keys and values of the step itself (prefill): rows of sequence s start at cu_rows[s] and stand at the
+    // positions from new_len[s] - count on (from 0 without new_len); row_pos holds every row's position
     const void* k; long k_stride; const void* v; long v_stride;
     const int* cu_rows; const int* row_seq; const int* row_pos;
-    // keys and values in the paged cache (decode): sequence i is row i, its last position new_len[i] - 1
+    // keys and values in the paged cache: all of them in a decode step (sequence i is row i, its last position
+    // new_len[i] - 1), the positions before the step's own rows otherwise
     const int* new_len; const int* table; int table_w; const void* k_pool; const void* v_pool; int page; int rows_cap;
     void* out;
     int H, KV, hd; float scale, cap; int window; int paged;
@@ -25,9 +27,13 @@ __global__ void __launch_bounds__(64)
 attn_simple_k(AttnSimpleArgs a) {
     const int h = blockIdx.y, r = blockIdx.x, lane = threadIdx.x;
     const int g = h / (a.H / a.KV);
-    int seq, p;
-    if (a.paged) { seq = r; p = a.new_len[r] - 1; }
-    else { seq = a.row_seq[r]; p = a.row_pos[r]; }
+    int seq, p, start = 0;                              // start: the first position that is a row of the step
+    if (a.paged) { seq = r; p = a.new_len[r] - 1; start = p + 1; }
+    else {
+        seq = a.row_seq[r];
+        p = a.row_pos[r];
+        if (a.new_len) start = a.new_len[seq] - (a.cu_rows[seq + 1] - a.cu_rows[seq]);
+    }
     const int lo = a.window > 0 ? max(0, p - a.window + 1) : 0;
     const T* q = (const T*)a.q + (size_t)r * a.q_stride + (size_t)h * a.hd;
     float qv[4], o[4];
@@ -43,14 +49,14 @@ attn_simple_k(AttnSimpleArgs a) {
     auto fetch = [&](int t, float (&kk)[4], float (&vv)[4]) {
         t = t < p ? t : p;                               // past the last key: a row that exists, never used
         const T *kp, *vp;
-        if (a.paged) {
+        if (t < start) {
             const int row = a.rows_cap > 0 ? t % a.rows_cap : t;
             const int pg = a.table[(size_t)seq * a.table_w + row / a.page];
             const size_t off = (((size_t)pg * a.KV + g) * a.page + row % a.page) * a.hd;
             kp = (const T*)a.k_pool + off;
             vp = (const T*)a.v_pool + off;
         } else {
-            const size_t row = (size_t)(a.cu_rows[seq] + t);
+            const size_t row = (size_t)(a.cu_rows[seq] + t - start);
             kp = (const T*)a.k + row * a.k_stride + (size_t)g * a.hd;
             vp = (const T*)a.v + row * a.v_stride + (size_t)g * a.hd;
         }
@@ -110,12 +116,19 @@ static int launch(const AttnSimpleArgs& a, int dtype, int M, hipStream_t s) {
     return tp_check_launch("attention (plain kernel)");
 }
 
+// new_len (or null): the sequences' lengths after the step; the positions before a sequence's first row of the step
+// are read from the cache (pools [pages, kv_heads, page, head_dim] through `table`), as earlier steps left it
 extern "C" int tp_attn_simple_prefill(const void* q, long q_stride, const void* k, long k_stride, const void* v, long v_stride,
                                       int dtype, int M, int H, int KV, int hd, const int* cu_rows, const int* row_seq,
-                                      const int* row_pos, float scale, float cap, int window, void* out, void* stream) {
+                                      const int* row_pos, const int* new_len, const int* table, int table_w,
+                                      const void* k_pool, const void* v_pool, int page, int rows_cap,
+                                      float scale, float cap, int window, void* out, void* stream) {
+    TP_REQUIRE(!new_len || (table && k_pool && v_pool && page > 0 && table_w > 0), "attention: cached positions need the page table and the pools");
     AttnSimpleArgs a{};
     a.q = q; a.q_stride = q_stride; a.k = k; a.k_stride = k_stride; a.v = v; a.v_stride = v_stride;
     a.cu_rows = cu_rows; a.row_seq = row_seq; a.row_pos = row_pos;
+    a.new_len = new_len; a.table = table; a.table_w = table_w; a.k_pool = k_pool; a.v_pool = v_pool;
+    a.page = new_len ? page : 1; a.rows_cap = new_len ? rows_cap : 0;
     a.out = out; a.H = H; a.KV = KV; a.hd = hd; a.scale = scale; a.cap = cap; a.window = window; a.paged = 0;
     return launch(a, dtype, M, (hipStream_t)stream);
 }

@@ -371,8 +371,8 @@ extern "C" int tp_gather_rows(const float* x, const int* rows, float* out, int n
 // A sequence's position p lives in row p (or p % rows_cap of a ring), found through its page list.
 // grid (rows, groups of heads): a block rotates `hpb` of the row's H + KV heads (query heads first); a thread
 // computes the cosine and sine of its pair once and applies them to all of them.  A key head goes into the
-// cache, with its value head, straight from registers; and, when the step gathers its visible keys into one
-// buffer (gk, gv: a sequence's position t in row key_row0[seq] + t), into that buffer as well.
+// cache, with its value head, straight from registers; without a page table the keys are rotated and nothing is
+// cached (a step whose attention still has to read the cache as earlier steps left it caches its rows afterwards).
 template <typename T>
 __global__ void __launch_bounds__(128)
 rope_kv_write_k(T* __restrict__ q, long q_stride, T* __restrict__ k, long k_stride,
@@ -380,16 +380,15 @@ rope_kv_write_k(T* __restrict__ q, long q_stride, T* __restrict__ k, long k_stri
                 const float* __restrict__ inv_freq, int rot,
                 const int* __restrict__ row_seq, const int* __restrict__ row_pos,
                 const int* __restrict__ new_len, const int* __restrict__ table, int table_w,
-                T* __restrict__ k_pool, T* __restrict__ v_pool, int page, int rows_cap, int hpb,
-                T* __restrict__ gk, T* __restrict__ gv, long g_stride, const int* __restrict__ key_row0, int pairing) {
+                T* __restrict__ k_pool, T* __restrict__ v_pool, int page, int rows_cap, int hpb, int pairing) {
     const int r = blockIdx.x;
     const int j_begin = blockIdx.y * hpb, j_end = min(j_begin + hpb, H + (k ? KV : 0));
     const int pos = row_pos[r];
     const int half = rot / 2;
     // where the row's keys and values go: the same page and row for every kv head
-    size_t cache_at = 0, gather_at = 0;
+    size_t cache_at = 0;
     bool cached = false;
-    if (k && j_end > H) {
+    if (k && table && j_end > H) {
         const int seq = row_seq[r];
         int row = pos;
         bool keep = true;
@@ -400,7 +399,6 @@ rope_kv_write_k(T* __restrict__ q, long q_stride, T* __restrict__ k, long k_stri
         const int pg = keep ? table[(size_t)seq * table_w + row / page] : -1;
         cached = pg >= 0;
         if (cached) cache_at = ((size_t)pg * KV * page + row % page) * hd;      // + kv head * page * hd
-        if (gk) gather_at = (size_t)(key_row0[seq] + pos) * g_stride;           // + kv head * hd
     }
     for (int f = threadIdx.x; f < half; f += blockDim.x) {     // one thread per pair: elements (f, f + half), or neighbours (2f, 2f + 1)
         const float ang = (float)pos * inv_freq[f];
@@ -422,24 +420,14 @@ rope_kv_write_k(T* __restrict__ q, long q_stride, T* __restrict__ k, long k_stri
                 v_pool[off + e0] = vsrc[e0];
                 v_pool[off + e1] = vsrc[e1];
             }
-            if (gk) {
-                const size_t off = gather_at + (size_t)(j - H) * hd;
-                st_f32(gk + off + e0, y0);
-                st_f32(gk + off + e1, y1);
-                gv[off + e0] = vsrc[e0];
-                gv[off + e1] = vsrc[e1];
-            }
         }
     }
-    if (cached || gk)
+    if (cached)
         for (int j = max(j_begin, H); j < j_end; j++) {           // elements outside the rotation
-            const size_t off = cache_at + (size_t)(j - H) * page * hd, goff = gather_at + (size_t)(j - H) * hd;
+            const size_t off = cache_at + (size_t)(j - H) * page * hd;
             const T* ksrc = k + (size_t)r * k_stride + (size_t)(j - H) * hd;
             const T* vsrc = v + (size_t)r * v_stride + (size_t)(j - H) * hd;
-            for (int d = rot + threadIdx.x; d < hd; d += blockDim.x) {
-                if (cached) { k_pool[off + d] = ksrc[d]; v_pool[off + d] = vsrc[d]; }
-                if (gk) { gk[goff + d] = ksrc[d]; gv[goff + d] = vsrc[d]; }
-            }
+            for (int d = rot + threadIdx.x; d < hd; d += blockDim.x) { k_pool[off + d] = ksrc[d]; v_pool[off + d] = vsrc[d]; }
         }
 }
 
@@ -452,8 +440,7 @@ rope_kv_write_vec_k(bf16_t* __restrict__ q, long q_stride, bf16_t* __restrict__ 
                     const float* __restrict__ inv_freq, int rot,
                     const int* __restrict__ row_seq, const int* __restrict__ row_pos,
                     const int* __restrict__ new_len, const int* __restrict__ table, int table_w,
-                    bf16_t* __restrict__ k_pool, bf16_t* __restrict__ v_pool, int page, int rows_cap,
-                    bf16_t* __restrict__ gk, bf16_t* __restrict__ gv, long g_stride, const int* __restrict__ key_row0) {
+                    bf16_t* __restrict__ k_pool, bf16_t* __restrict__ v_pool, int page, int rows_cap) {
     __shared__ float cs[128], sn[128];
     const int r = blockIdx.x, pos = row_pos[r], half = rot / 2;
     for (int f = threadIdx.x; f < half; f += 256) {
@@ -461,9 +448,9 @@ rope_kv_write_vec_k(bf16_t* __restrict__ q, long q_stride, bf16_t* __restrict__ 
         cs[f] = cosf(ang);
         sn[f] = sinf(ang);
     }
-    size_t cache_at = 0, gather_at = 0;
+    size_t cache_at = 0;
     bool cached = false;
-    if (k) {
+    if (k && table) {
         const int seq = row_seq[r];
         int row = pos;
         bool keep = true;
@@ -474,7 +461,6 @@ rope_kv_write_vec_k(bf16_t* __restrict__ q, long q_stride, bf16_t* __restrict__ 
         const int pg = keep ? table[(size_t)seq * table_w + row / page] : -1;
         cached = pg >= 0;
         if (cached) cache_at = ((size_t)pg * KV * page + row % page) * hd;      // + kv head * page * hd
-        if (gk) gather_at = (size_t)(key_row0[seq] + pos) * g_stride;           // + kv head * hd
     }
     __syncthreads();
     union Piece { uint4 u; bf16_t h[8]; };
@@ -504,30 +490,16 @@ rope_kv_write_vec_k(bf16_t* __restrict__ q, long q_stride, bf16_t* __restrict__ 
             *reinterpret_cast<uint4*>(v_pool + off + f0) = v0;
             *reinterpret_cast<uint4*>(v_pool + off + f0 + half) = v1;
         }
-        if (gk) {
-            const size_t off = gather_at + (size_t)(j - H) * hd;
-            *reinterpret_cast<uint4*>(gk + off + f0) = lo.u;
-            *reinterpret_cast<uint4*>(gk + off + f0 + half) = hi.u;
-            *reinterpret_cast<uint4*>(gv + off + f0) = v0;
-            *reinterpret_cast<uint4*>(gv + off + f0 + half) = v1;
-        }
     }
-    if (k && (cached || gk)) {                                    // elements outside the rotation
+    if (cached) {                                                 // elements outside the rotation
         const int rest = (hd - rot) / 8;
         for (int item = threadIdx.x; item < KV * rest; item += 256) {
             const int j = item / rest, d = rot + (item - j * rest) * 8;
             const uint4 kk = *reinterpret_cast<const uint4*>(k + (size_t)r * k_stride + (size_t)j * hd + d);
             const uint4 vv = *reinterpret_cast<const uint4*>(v + (size_t)r * v_stride + (size_t)j * hd + d);
-            if (cached) {
-                const size_t off = cache_at + (size_t)j * page * hd + d;
-                *reinterpret_cast<uint4*>(k_pool + off) = kk;
-                *reinterpret_cast<uint4*>(v_pool + off) = vv;
-            }
-            if (gk) {
-                const size_t off = gather_at + (size_t)j * hd + d;
-                *reinterpret_cast<uint4*>(gk + off) = kk;
-                *reinterpret_cast<uint4*>(gv + off) = vv;
-            }
+            const size_t off = cache_at + (size_t)j * page * hd + d;
+            *reinterpret_cast<uint4*>(k_pool + off) = kk;
+            *reinterpret_cast<uint4*>(v_pool + off) = vv;
         }
     }
 }
@@ -536,26 +508,25 @@ extern "C" int tp_rope_kv_write(void* q, long q_stride, void* k, long k_stride, 
                                 int dtype, int M, int H, int KV, int hd, const float* inv_freq, int rot,
                                 const int* row_seq, const int* row_pos, const int* new_len,
                                 const int* table, int table_w, void* k_pool, void* v_pool,
-                                int page, int rows_cap, void* gk, void* gv, long g_stride, const int* key_row0,
-                                int pairing, void* stream) {
+                                int page, int rows_cap, int pairing, void* stream) {
     TP_REQUIRE(M > 0 && H > 0 && hd > 0, "rope_kv_write: empty shape M=%d H=%d hd=%d", M, H, hd);
     TP_REQUIRE(rot >= 0 && rot <= hd && rot % 2 == 0, "rope_kv_write: rotary_dim %d must be even and at most head_dim %d", rot, hd);
     TP_REQUIRE(rot == 0 || inv_freq, "rope_kv_write: a rotation needs its frequency table");
     TP_REQUIRE(pairing == TP_ROPE_HALVES || pairing == TP_ROPE_NEIGHBOURS, "rope_kv_write: pairing %d is neither halves (%d) nor neighbours (%d)",
                pairing, TP_ROPE_HALVES, TP_ROPE_NEIGHBOURS);
-    TP_REQUIRE(!k || (v && k_pool && v_pool && table && KV > 0 && page > 0 && table_w > 0),
-               "rope_kv_write: keys without values, cache pools or page table");
+    // table null: the keys are rotated and nothing is cached
+    TP_REQUIRE(!k || (v && KV > 0), "rope_kv_write: keys without values");
+    TP_REQUIRE(!k || !table || (k_pool && v_pool && page > 0 && table_w > 0), "rope_kv_write: a page table without cache pools");
+    if (!table) { page = 1; rows_cap = 0; }
     TP_REQUIRE(rows_cap >= 0 && (rows_cap == 0 || rows_cap % page == 0), "rope_kv_write: ring of %d rows is no multiple of the page size %d", rows_cap, page);
-    TP_REQUIRE(!gk || (k && gv && key_row0 && g_stride >= (long)KV * hd), "rope_kv_write: a gathered copy needs keys, both buffers, their rows' origin and rows of at least %ld elements", (long)KV * hd);
     hipStream_t s = (hipStream_t)stream;
     TP_REQUIRE(H + KV <= 65535, "rope_kv_write: %d heads exceed one launch", H + KV);
     const int heads = H + (k ? KV : 0);
     auto piecewise = [](const void* p, long stride) { return !p || ((uintptr_t)p % 16 == 0 && stride % 8 == 0); };
     if (pairing == TP_ROPE_HALVES && dtype == TP_BF16 && M >= 256 && hd % 8 == 0 && rot % 16 == 0 && rot <= 256 && piecewise(q, q_stride) && piecewise(k, k_stride) &&
-        piecewise(v, v_stride) && piecewise(k_pool, 8) && piecewise(v_pool, 8) && piecewise(gk, g_stride) && piecewise(gv, g_stride)) {
+        piecewise(v, v_stride) && piecewise(k_pool, 8) && piecewise(v_pool, 8)) {
         rope_kv_write_vec_k<<<M, 256, 0, s>>>((bf16_t*)q, q_stride, (bf16_t*)k, k_stride, (const bf16_t*)v, v_stride, H, KV, hd,
-            inv_freq, rot, row_seq, row_pos, new_len, table, table_w, (bf16_t*)k_pool, (bf16_t*)v_pool, page, rows_cap,
-            (bf16_t*)gk, (bf16_t*)gv, g_stride, key_row0);
+            inv_freq, rot, row_seq, row_pos, new_len, table, table_w, (bf16_t*)k_pool, (bf16_t*)v_pool, page, rows_cap);
         return tp_check_launch("rope_kv_write");
     }
     // many rows: one block per row shares each pair's cosine and sine over all heads; few rows: a block per head
@@ -564,62 +535,69 @@ extern "C" int tp_rope_kv_write(void* q, long q_stride, void* k, long k_stride, 
     const int threads = hd <= 64 ? 64 : 128;
     if (dtype == TP_BF16)
         rope_kv_write_k<bf16_t><<<grid, threads, 0, s>>>((bf16_t*)q, q_stride, (bf16_t*)k, k_stride, (const bf16_t*)v, v_stride, H, KV, hd,
-            inv_freq, rot, row_seq, row_pos, new_len, table, table_w, (bf16_t*)k_pool, (bf16_t*)v_pool, page, rows_cap, hpb,
-            (bf16_t*)gk, (bf16_t*)gv, g_stride, key_row0, pairing);
+            inv_freq, rot, row_seq, row_pos, new_len, table, table_w, (bf16_t*)k_pool, (bf16_t*)v_pool, page, rows_cap, hpb, pairing);
     else if (dtype == TP_F32)
         rope_kv_write_k<float><<<grid, threads, 0, s>>>((float*)q, q_stride, (float*)k, k_stride, (const float*)v, v_stride, H, KV, hd,
-            inv_freq, rot, row_seq, row_pos, new_len, table, table_w, (float*)k_pool, (float*)v_pool, page, rows_cap, hpb,
-            (float*)gk, (float*)gv, g_stride, key_row0, pairing);
+            inv_freq, rot, row_seq, row_pos, new_len, table, table_w, (float*)k_pool, (float*)v_pool, page, rows_cap, hpb, pairing);
     else return tp_fail("rope_kv_write: unknown dtype %d", dtype);
     return tp_check_launch("rope_kv_write");
 }
 
-// ---- the cached keys and values a step's queries see, copied out of the paged cache ----------------------------
-// A step that continues sequences by several tokens attends over one buffer per cache group: each sequence's
-// cached positions prefix_lo[s] .. start[s] - 1 (copied here, before the step writes its own rows into a ring that
-// may overwrite them), then the step's own rows (rope_kv_write adds them).  Sequence s's position t goes to row
-// cu_keys[s] + t - prefix_lo[s].  grid (cached position, sequence); a block copies the row's kv heads of K and V.
+// ---- a step's keys (rotated already) and values into the paged cache ------------------------------------------------
+// For steps whose attention reads the cache as earlier steps left it and therefore caches its own rows afterwards: in a
+// ring without a row to spare the step's rows take the places of positions that its earlier queries still see.
+// grid (rows); a block copies the row's kv heads of K and V; of rows that share a ring row the last one stays.
 template <typename T>
 __global__ void __launch_bounds__(256)
-gather_kv_prefix_k(const T* __restrict__ k_pool, const T* __restrict__ v_pool, const int* __restrict__ table, int table_w,
-                   int page, int rows_cap, int KV, int hd, const int* __restrict__ cu_rows, const int* __restrict__ cu_keys,
-                   const int* __restrict__ prefix_lo, T* __restrict__ gk, T* __restrict__ gv, long g_stride) {
-    const int seq = blockIdx.y, j = blockIdx.x;
-    const int cached = (cu_keys[seq + 1] - cu_keys[seq]) - (cu_rows[seq + 1] - cu_rows[seq]);
-    if (j >= cached) return;
-    const int t = prefix_lo[seq] + j;
-    const int row = rows_cap > 0 ? t % rows_cap : t;
+kv_write_k(const T* __restrict__ k, long k_stride, const T* __restrict__ v, long v_stride, int KV, int hd,
+           const int* __restrict__ row_seq, const int* __restrict__ row_pos, const int* __restrict__ new_len,
+           const int* __restrict__ table, int table_w, T* __restrict__ k_pool, T* __restrict__ v_pool, int page, int rows_cap) {
+    const int r = blockIdx.x, seq = row_seq[r], pos = row_pos[r];
+    int row = pos;
+    if (rows_cap > 0) {
+        if (pos + rows_cap < new_len[seq]) return;       // a later row of this step takes the same ring row
+        row = pos % rows_cap;
+    }
     const int pg = table[(size_t)seq * table_w + row / page];
-    if (pg < 0) return;                                  // never for a position the cache holds
-    const size_t dst = (size_t)(cu_keys[seq] + j) * g_stride;
-    for (int i = threadIdx.x; i < KV * hd; i += blockDim.x) {
-        const int g = i / hd, d = i - g * hd;
-        const size_t src = (((size_t)pg * KV + g) * page + row % page) * hd + d;
-        gk[dst + i] = k_pool[src];
-        gv[dst + i] = v_pool[src];
+    if (pg < 0) return;                                  // never for a position the cache has room for
+    const size_t at = ((size_t)pg * KV * page + row % page) * hd;
+    constexpr int PIECE = 16 / sizeof(T);                // elements of a 16-byte piece
+    const bool wide = hd % PIECE == 0 && k_stride % PIECE == 0 && v_stride % PIECE == 0 && (uintptr_t)k % 16 == 0 &&
+                      (uintptr_t)v % 16 == 0 && (uintptr_t)k_pool % 16 == 0 && (uintptr_t)v_pool % 16 == 0;
+    if (wide) {
+        const int per_head = hd / PIECE;
+        for (int i = threadIdx.x; i < KV * per_head; i += blockDim.x) {
+            const int g = i / per_head, d = (i - g * per_head) * PIECE;
+            const size_t dst = at + (size_t)g * page * hd + d;
+            *reinterpret_cast<uint4*>(k_pool + dst) = *reinterpret_cast<const uint4*>(k + (size_t)r * k_stride + (size_t)g * hd + d);
+            *reinterpret_cast<uint4*>(v_pool + dst) = *reinterpret_cast<const uint4*>(v + (size_t)r * v_stride + (size_t)g * hd + d);
+        }
+    } else {
+        for (int i = threadIdx.x; i < KV * hd; i += blockDim.x) {
+            const int g = i / hd, d = i - g * hd;
+            const size_t dst = at + (size_t)g * page * hd + d;
+            k_pool[dst] = k[(size_t)r * k_stride + i];
+            v_pool[dst] = v[(size_t)r * v_stride + i];
+        }
     }
 }
 
-extern "C" int tp_gather_kv_prefix(const void* k_pool, const void* v_pool, int dtype, const int* table, int table_w,
-                                   int page, int rows_cap, int KV, int hd, int n_seq, const int* cu_rows,
-                                   const int* cu_keys, const int* prefix_lo, int max_prefix,
-                                   void* gk, void* gv, long g_stride, void* stream) {
-    TP_REQUIRE(n_seq > 0 && KV > 0 && hd > 0 && page > 0 && table_w > 0, "gather_kv_prefix: empty shape");
-    TP_REQUIRE(k_pool && v_pool && table && cu_rows && cu_keys && prefix_lo && gk && gv, "gather_kv_prefix: a null operand");
-    TP_REQUIRE(rows_cap >= 0 && (rows_cap == 0 || rows_cap % page == 0), "gather_kv_prefix: ring of %d rows is no multiple of the page size %d", rows_cap, page);
-    TP_REQUIRE(g_stride >= (long)KV * hd, "gather_kv_prefix: rows of %ld elements are too short for %d heads of %d", g_stride, KV, hd);
-    TP_REQUIRE(n_seq <= 65535, "gather_kv_prefix: %d sequences exceed one launch", n_seq);
-    if (max_prefix <= 0) return 0;
-    dim3 grid(max_prefix, n_seq);
+extern "C" int tp_kv_write(const void* k, long k_stride, const void* v, long v_stride, int dtype, int M, int KV, int hd,
+                           const int* row_seq, const int* row_pos, const int* new_len, const int* table, int table_w,
+                           void* k_pool, void* v_pool, int page, int rows_cap, void* stream) {
+    TP_REQUIRE(M > 0 && KV > 0 && hd > 0 && page > 0 && table_w > 0, "kv_write: empty shape");
+    TP_REQUIRE(k && v && row_seq && row_pos && new_len && table && k_pool && v_pool, "kv_write: a null operand");
+    TP_REQUIRE(k_stride >= (long)KV * hd && v_stride >= (long)KV * hd, "kv_write: rows are too short for %d heads of %d", KV, hd);
+    TP_REQUIRE(rows_cap >= 0 && (rows_cap == 0 || rows_cap % page == 0), "kv_write: ring of %d rows is no multiple of the page size %d", rows_cap, page);
     hipStream_t s = (hipStream_t)stream;
     if (dtype == TP_BF16)
-        gather_kv_prefix_k<bf16_t><<<grid, 256, 0, s>>>((const bf16_t*)k_pool, (const bf16_t*)v_pool, table, table_w, page, rows_cap,
-            KV, hd, cu_rows, cu_keys, prefix_lo, (bf16_t*)gk, (bf16_t*)gv, g_stride);
+        kv_write_k<bf16_t><<<M, 256, 0, s>>>((const bf16_t*)k, k_stride, (const bf16_t*)v, v_stride, KV, hd, row_seq, row_pos, new_len,
+                                             table, table_w, (bf16_t*)k_pool, (bf16_t*)v_pool, page, rows_cap);
     else if (dtype == TP_F32)
-        gather_kv_prefix_k<float><<<grid, 256, 0, s>>>((const float*)k_pool, (const float*)v_pool, table, table_w, page, rows_cap,
-            KV, hd, cu_rows, cu_keys, prefix_lo, (float*)gk, (float*)gv, g_stride);
-    else return tp_fail("gather_kv_prefix: unknown dtype %d", dtype);
-    return tp_check_launch("gather_kv_prefix");
+        kv_write_k<float><<<M, 256, 0, s>>>((const float*)k, k_stride, (const float*)v, v_stride, KV, hd, row_seq, row_pos, new_len,
+                                            table, table_w, (float*)k_pool, (float*)v_pool, page, rows_cap);
+    else return tp_fail("kv_write: unknown dtype %d", dtype);
+    return tp_check_launch("kv_write");
 }
 
 // ---- gated activation on a packed gate/up product: y [M, 2*Ip] fp32 with 16 gate columns, then the 16 up

@@ -30,24 +30,7 @@ def classify(counts, starts):
     return "extend"
 
 
-class KeyGeometry:
-    """Where a sequence's visible keys lie when a step gathers them into one buffer per cache group: the cached
-    positions prefix_lo[i] .. start[i] - 1 (all of them, or the last window - 1), then the step's own rows.
-    Sequence i's keys are rows cu_keys[i] .. cu_keys[i + 1] - 1, position t in row key_row0[i] + t."""
-
-    def __init__(self, starts, counts, window):
-        starts, counts = np.asarray(starts, dtype=np.int64), np.asarray(counts, dtype=np.int64)
-        self.prefix_lo = np.maximum(0, starts - (window - 1)) if window else np.zeros_like(starts)
-        keys = starts - self.prefix_lo + counts
-        self.cu_keys = np.zeros(len(starts) + 1, dtype=np.int64)
-        np.cumsum(keys, out=self.cu_keys[1:])
-        self.key_row0 = self.cu_keys[:-1] - self.prefix_lo
-        self.total_keys = int(self.cu_keys[-1])
-        self.max_keys = int(keys.max())
-        self.max_prefix = int((starts - self.prefix_lo).max())
-
-
-def step_arrays(cache, slots, counts, starts, want_rows, table_widths=None, key_geometry=()):
+def step_arrays(cache, slots, counts, starts, want_rows, table_widths=None):
     """The step's geometry as int32 arrays, in the order StepContext slices them."""
     n, m = len(slots), int(sum(counts))
     cu = np.zeros(n + 1, dtype=np.int64)
@@ -64,8 +47,6 @@ def step_arrays(cache, slots, counts, starts, want_rows, table_widths=None, key_
         t = cache.page_table(gi, slots, None if table_widths is None else table_widths[gi])
         shapes.append(t.shape)
         parts.append(t.reshape(-1))
-    for g in key_geometry:
-        parts.extend([g.cu_keys, g.key_row0, g.prefix_lo])
     flat = np.concatenate([np.asarray(p, dtype=np.int32).reshape(-1) for p in parts])
     return flat, shapes
 
@@ -134,11 +115,9 @@ class StepContext:
         self._shared = set()            # entries whose step keys/values a later entry reads
         self._step_kv = {}
         n, m = self.n_seq, self.n_rows
-        self.key_geometry = []
-        if self.mode == "extend":
-            self.key_geometry = [KeyGeometry(self.starts, self.counts, g.spec.window) for g in cache.kv_groups]
+        self._after_step = []           # work put off until every entry of the step has run
         flat, shapes = step_arrays(cache, self.slots, self.counts, self.starts, want_rows,
-                                   static.table_widths if static is not None else None, self.key_geometry)
+                                   static.table_widths if static is not None else None)
         if static is not None:
             dev = static.device_buffer
         else:
@@ -159,8 +138,6 @@ class StepContext:
         self.identity_want = list(want_rows) == list(range(m))
         self.want_rows = take(self.n_want)
         self._tables = [take(int(np.prod(sh))).reshape(sh) for sh in shapes]
-        for g in self.key_geometry:          # the same numbers on the device
-            g.cu_keys_dev, g.key_row0_dev, g.prefix_lo_dev = take(n + 1), take(n), take(n)
 
     def page_table(self, group_index):
         return self._tables[group_index]
@@ -176,10 +153,6 @@ class StepContext:
         print(f"[ldump] L={-1 if self.entry is None else self.entry} stage={stage} l2={float(t.norm()):.6e} "
               f"absmax={float(t.abs().max()):.6e} mean={float(t.mean()):.6e}", file=sys.stderr, flush=True)
 
-    def keys_of(self, group_index):
-        """The KeyGeometry of a cache group in an "extend" step (host arrays, and `*_dev` int32 on the device)."""
-        return self.key_geometry[group_index]
-
     def max_keys(self, site):
         """Most keys any sequence of this step can see at this cache site (a host number, for launch geometry).
         With fixed step memory (a captured graph) it is the graph's bound on the lengths."""
@@ -193,9 +166,23 @@ class StepContext:
         self._shared = set(entries)
 
     def offer_step_kv(self, k, v):
-        """k, v: the rows this step's attention reads (the step's own, or in an "extend" step the gathered ones)."""
+        """k, v: this step's own rows of the running entry, for the entries that read its cache."""
         if self.entry in self._shared:
             self._step_kv[self.entry] = (k, v)
 
     def step_kv_of(self, entry):
         return self._step_kv[entry]
+
+    def after_readers(self, work):
+        """Run `work()` once nobody in this step reads the running entry's cache as earlier steps left it any more:
+        at once, or at the end of the step when later entries read this entry's cache."""
+        if self.entry in self._shared:
+            self._after_step.append(work)
+        else:
+            work()
+
+    def finish(self):
+        """What was put off until the end of the step."""
+        for work in self._after_step:
+            work()
+        self._after_step = []

@@ -171,6 +171,7 @@ class Model:
                 next_norm = None
             stream, normed = self.layers[e.layer].block.forward(ctx, stream, cache.site(ctx.cache_owner),
                                                                  normed=normed, next_norm=next_norm)
+        ctx.finish()
         if ctx.n_want == 0:
             return None
         if whole and normed is not None:

@@ -19,7 +19,7 @@ ARCH = "gfx950"
 FLAGS = ["--offload-arch=" + ARCH, "-O3", "-fPIC", "-std=c++17",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-result"]
 CORE_SOURCES = ["elementwise.hip", "gemm.hip", "gemm_skinny.hip", "gemm_mfma.hip", "gemv.hip", "gemm_rows8.hip", "attention_simple.hip", "sampling.hip", "probes.hip"]
-ATTN_SOURCE = "attention_mfma.hip"
+ATTN_SOURCES = ["attention_mfma.hip", "attention_prefill.hip"]      # decode steps; steps of many queries
 _NOISE = "is not a recognized feature for this target"
 
 
@@ -146,4 +146,4 @@ def attn_name(head_dim):
 
 
 def build_attention(head_dim, force=False):
-    return build_library(attn_name(head_dim), [ATTN_SOURCE], [f"-DTP_HD={head_dim}"], force=force)
+    return build_library(attn_name(head_dim), ATTN_SOURCES, [f"-DTP_HD={head_dim}"], force=force)

@@ -19,13 +19,12 @@ _CORE_SIGS = {
     "tp_add_rms_norm": [_P, _P, _I, _I, _L, _P, _F, _P, _F, _P, _I, _I, _I, _P],
     "tp_gather_rows": [_P, _P, _P, _I, _I, _I, _P],
     "tp_sum_slices": [_P, _I, _L, _P, _I, _L, _P],
-    "tp_rope_kv_write": [_P, _L, _P, _L, _P, _L, _I, _I, _I, _I, _I, _P, _I, _P, _P, _P, _P, _I, _P, _P, _I, _I,
-                         _P, _P, _L, _P, _I, _P],
-    "tp_gather_kv_prefix": [_P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P, _P, _P, _I, _P, _P, _L, _P],
+    "tp_rope_kv_write": [_P, _L, _P, _L, _P, _L, _I, _I, _I, _I, _I, _P, _I, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _P],
+    "tp_kv_write": [_P, _L, _P, _L, _I, _I, _I, _I, _P, _P, _P, _P, _I, _P, _P, _I, _I, _P],
     "tp_gated_act": [_P, _P, _I, _I, _I, _I, _P],
     "tp_linear": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P, _L, _I, _I, _P],
     "tp_linear_workspace_bytes": [_I, _I, _I, _I, _I, _I, _I, _I, _I],
-    "tp_attn_simple_prefill": [_P, _L, _P, _L, _P, _L, _I, _I, _I, _I, _I, _P, _P, _P, _F, _F, _I, _P, _P],
+    "tp_attn_simple_prefill": [_P, _L, _P, _L, _P, _L, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _F, _F, _I, _P, _P],
     "tp_attn_simple_decode": [_P, _L, _I, _I, _I, _I, _I, _P, _P, _I, _P, _P, _I, _I, _F, _F, _I, _P, _P],
     "tp_argmax": [_P, _I, _I, _P, _P, _P],
     "tp_argmax_workspace_bytes": [_I, _I],
@@ -38,8 +37,7 @@ _CORE_SIGS = {
     "tp_probe_mfma": [_I, _I, _I, _P, _P, _P],
 }
 _ATTN_SIGS = {
-    "tp_attn_prefill": [_P, _L, _P, _L, _P, _L, _I, _I, _I, _P, _I, _I, _P, _I, _I, _F, _F, _I, _P, _P, _P],
-    "tp_attn_prefill_workspace_elems": [_I, _I, _I],
+    "tp_attn_prefill": [_P, _L, _P, _L, _P, _L, _I, _I, _I, _P, _I, _I, _P, _P, _I, _P, _P, _I, _I, _F, _F, _I, _P, _I, _P],
     "tp_attn_decode": [_P, _L, _I, _I, _I, _P, _P, _I, _P, _P, _I, _I, _F, _F, _I, _P, _P, _I, _P],
     "tp_attn_decode_workspace_floats": [_I, _I, _I],
     "tp_attn_decode_fused": [_P, _I, _I, _L, _L, _P, _I, _I, _I, _I, _I, _P, _P, _I, _P, _P, _I, _I, _F, _F, _I, _P, _P, _I, _P],
@@ -245,9 +243,9 @@ class HipOps:
         return out
 
     def rope_kv_write(self, q, k, v, H, KV, hd, inv_freq, rotary_dim, row_seq, row_pos, new_len, table,
-                      k_pool, v_pool, rows_cap, gathered=None, pairing="halves"):
-        """Rotate q and k in place and write k, v into the cache.  gathered = (gk, gv, key_row0): the step's rows
-        also go into the buffers that `gather_kv_prefix` began, position t of sequence s into row key_row0[s] + t.
+                      k_pool, v_pool, rows_cap, pairing="halves", write=True):
+        """Rotate q and k in place and write k, v into the cache.  write=False: rotate only (a step whose attention
+        reads the cache as earlier steps left it caches its rows afterwards, with `kv_write`).
         pairing: one of ROPE_PAIRINGS, which elements of a head turn together."""
         if pairing not in ROPE_PAIRINGS:
             raise KernelError(f"rope_kv_write: pairing '{pairing}' has no kernel ({', '.join(ROPE_PAIRINGS)})")
@@ -264,55 +262,35 @@ class HipOps:
                 raise KernelError("rope_kv_write: row_seq and row_pos must be int32, one entry per row")
         kp = vp = ks = vs = 0
         page = table_w = 1
+        write = write and k is not None
         if k is not None:
             ks, vs = self._rows(k, "rope_kv_write k"), self._rows(v, "rope_kv_write v")
             if k.shape != (m, KV * hd) or v.shape != (m, KV * hd) or k.dtype != q.dtype or v.dtype != q.dtype:
                 raise KernelError("rope_kv_write: k and v must be [rows, kv_heads * head_dim] of q's dtype")
-            if k_pool.dtype != q.dtype or k_pool.dim() != 4 or tuple(k_pool.shape[1:]) != (KV, k_pool.shape[2], hd) \
-                    or v_pool.shape != k_pool.shape or not k_pool.is_contiguous() or not v_pool.is_contiguous():
-                raise KernelError("rope_kv_write: cache pools must be contiguous [pages, kv_heads, page, head_dim] of q's dtype")
-            if table.dtype != torch.int32 or table.dim() != 2 or not table.is_contiguous() or table.shape[0] != new_len.numel():
-                raise KernelError("rope_kv_write: the page table must be contiguous int32 [sequences, pages]")
-            page, table_w = k_pool.shape[2], table.shape[1]
             kp, vp = k.data_ptr(), v.data_ptr()
-        gk = gv = row0 = None
-        g_stride = 0
-        if gathered is not None:
-            gk, gv, row0 = gathered
-            self._dev(gk, gv, row0)
-            if k is None or gk.dtype != q.dtype or gv.dtype != q.dtype or gk.shape != gv.shape or gk.dim() != 2 \
-                    or gk.shape[1] != KV * hd or not gk.is_contiguous() or not gv.is_contiguous():
-                raise KernelError("rope_kv_write: the gathered buffers must be contiguous [keys, kv_heads * head_dim] of q's dtype")
-            if row0.dtype != torch.int32 or row0.numel() != new_len.numel():
-                raise KernelError("rope_kv_write: one int32 row origin per sequence")
-            g_stride = gk.stride(0)
+        if write:
+            self._check_pools("rope_kv_write", q.dtype, new_len.numel(), KV, hd, new_len, table, k_pool, v_pool)
+            page, table_w = k_pool.shape[2], table.shape[1]
         self._call(self.lib, "tp_rope_kv_write", q.data_ptr(), qs, kp or None, ks, vp or None, vs, _code(q.dtype), m, H, KV, hd,
                    inv_freq.data_ptr() if rotary_dim else None, rotary_dim, row_seq.data_ptr(), row_pos.data_ptr(),
-                   new_len.data_ptr(), table.data_ptr() if k is not None else None, table_w,
-                   k_pool.data_ptr() if k is not None else None, v_pool.data_ptr() if k is not None else None,
-                   page, rows_cap, gk.data_ptr() if gk is not None else None, gv.data_ptr() if gv is not None else None,
-                   g_stride, row0.data_ptr() if row0 is not None else None, ROPE_PAIRINGS[pairing], self._stream())
+                   new_len.data_ptr(), table.data_ptr() if write else None, table_w,
+                   k_pool.data_ptr() if write else None, v_pool.data_ptr() if write else None,
+                   page, rows_cap if write else 0, ROPE_PAIRINGS[pairing], self._stream())
 
-    def gather_kv_prefix(self, table, k_pool, v_pool, rows_cap, cu_rows, keys):
-        """Buffers gk, gv [keys.total_keys, kv_heads * head_dim] with every sequence's cached positions
-        keys.prefix_lo[s] .. start[s] - 1 copied out of the cache (sequence s's position t in row keys.key_row0[s] + t);
-        the rows of the step itself are left for `rope_kv_write(..., gathered=)`.  keys: the step's KeyGeometry."""
-        self._dev(table, k_pool, v_pool, cu_rows, keys.cu_keys_dev, keys.prefix_lo_dev)
-        n = table.shape[0]
-        if k_pool.dim() != 4 or v_pool.shape != k_pool.shape or not k_pool.is_contiguous() or not v_pool.is_contiguous():
-            raise KernelError("gather_kv_prefix: cache pools must be contiguous [pages, kv_heads, page, head_dim]")
-        if table.dtype != torch.int32 or table.dim() != 2 or not table.is_contiguous():
-            raise KernelError("gather_kv_prefix: the page table must be contiguous int32 [sequences, pages]")
-        for t, size in ((cu_rows, n + 1), (keys.cu_keys_dev, n + 1), (keys.prefix_lo_dev, n)):
-            if t.dtype != torch.int32 or t.numel() != size:
-                raise KernelError("gather_kv_prefix: the step's geometry must be int32 arrays over its sequences")
-        _, KV, page, hd = k_pool.shape
-        gk = torch.empty((keys.total_keys, KV * hd), dtype=k_pool.dtype, device=self.device)
-        gv = torch.empty_like(gk)
-        self._call(self.lib, "tp_gather_kv_prefix", k_pool.data_ptr(), v_pool.data_ptr(), _code(k_pool.dtype), table.data_ptr(),
-                   table.shape[1], page, rows_cap, KV, hd, n, cu_rows.data_ptr(), keys.cu_keys_dev.data_ptr(),
-                   keys.prefix_lo_dev.data_ptr(), int(keys.max_prefix), gk.data_ptr(), gv.data_ptr(), gk.stride(0), self._stream())
-        return gk, gv
+    def kv_write(self, k, v, KV, hd, row_seq, row_pos, new_len, table, k_pool, v_pool, rows_cap):
+        """The step's keys (rotated already) and values into the cache: what `rope_kv_write(write=False)` left undone."""
+        self._dev(k, v, row_seq, row_pos, new_len, table, k_pool, v_pool)
+        m = k.shape[0]
+        ks, vs = self._rows(k, "kv_write k"), self._rows(v, "kv_write v")
+        if k.shape != (m, KV * hd) or v.shape != (m, KV * hd) or k.dtype != v.dtype:
+            raise KernelError("kv_write: k and v must be [rows, kv_heads * head_dim] of one dtype")
+        for t in (row_seq, row_pos):
+            if t.dtype != torch.int32 or t.numel() != m:
+                raise KernelError("kv_write: row_seq and row_pos must be int32, one entry per row")
+        self._check_pools("kv_write", k.dtype, new_len.numel(), KV, hd, new_len, table, k_pool, v_pool)
+        self._call(self.lib, "tp_kv_write", k.data_ptr(), ks, v.data_ptr(), vs, _code(k.dtype), m, KV, hd, row_seq.data_ptr(),
+                   row_pos.data_ptr(), new_len.data_ptr(), table.data_ptr(), table.shape[1], k_pool.data_ptr(),
+                   v_pool.data_ptr(), k_pool.shape[2], rows_cap, self._stream())
 
     # ---- matrix products -----------------------------------------------------------------------------
     def _linear(self, x, w, out_dtype, epilogue, cap, units, defer=False, act=0):
@@ -369,38 +347,45 @@ class HipOps:
         return not self.force_plain_attention and dtype == torch.bfloat16 and hd % 16 == 0 and hd <= 256 and H // KV <= 16
 
     def attention_prefill(self, q, k, v, H, KV, hd, cu_rows, max_count, scale, softcap, window, out_dtype,
-                          row_seq=None, row_pos=None, keys=None):
-        """Causal attention of the step's queries over rows of keys and values: the step's own (every sequence
-        starts: row_pos counts from 0), or with `keys` (a KeyGeometry) the gathered buffers, in which sequence s's
-        position t is row keys.key_row0[s] + t and row_pos holds absolute positions."""
+                          row_seq=None, row_pos=None, cached=None, shape=0):
+        """Causal attention of the step's queries over the step's own rows of keys and values and, with
+        `cached` = (new_len, table, k_pool, v_pool, rows_cap), over the positions before them, read in place from the
+        cache as earlier steps left it (the step's own rows are not looked for there).  Without `cached` every sequence
+        starts at position 0; with it row_pos holds absolute positions, sequence s's first row standing at
+        new_len[s] - its count.  shape: the matrix-core kernel's block shape (0: chosen by the size of the step)."""
         self._dev(q, k, v, cu_rows)
         m = q.shape[0]
-        mk = m if keys is None else keys.total_keys
         qs, ks, vs = self._rows(q, "attention q"), self._rows(k, "attention k"), self._rows(v, "attention v")
-        if q.shape[1] != H * hd or k.shape != (mk, KV * hd) or v.shape != (mk, KV * hd):
-            raise KernelError("attention_prefill: q must be [rows, heads * head_dim], k and v [keys, kv_heads * head_dim]")
+        if q.shape[1] != H * hd or k.shape != (m, KV * hd) or v.shape != (m, KV * hd):
+            raise KernelError("attention_prefill: q must be [rows, heads * head_dim], k and v [rows, kv_heads * head_dim]")
         if not (q.dtype == k.dtype == v.dtype == out_dtype):
             raise KernelError("attention_prefill: q, k, v and the output share one dtype")
         n_seq = cu_rows.numel() - 1
+        new_len = table = k_pool = v_pool = None
+        page, rows_cap, table_w = 1, 0, 1
+        if cached is not None:
+            new_len, table, k_pool, v_pool, rows_cap = cached
+            self._dev(new_len, table, k_pool, v_pool)
+            self._check_pools("attention_prefill", q.dtype, n_seq, KV, hd, new_len, table, k_pool, v_pool)
+            page, table_w, rows_cap = k_pool.shape[2], table.shape[1], rows_cap or 0
+        ptr = lambda t: t.data_ptr() if t is not None else None
         out = torch.empty((m, H * hd), dtype=out_dtype, device=self.device)
-        if self._fast_attention(q.dtype, H, KV, hd):
+        if self._fast_attention(q.dtype, H, KV, hd) and (cached is None or (page >= 16 and page & (page - 1) == 0)):
             lib = self.attn_lib(hd)
-            ws = torch.empty(lib.tp_attn_prefill_workspace_elems(mk, KV, n_seq), dtype=torch.bfloat16, device=self.device)
             self._call(lib, "tp_attn_prefill", q.data_ptr(), qs, k.data_ptr(), ks, v.data_ptr(), vs,
-                       m, H, KV, cu_rows.data_ptr(), n_seq, int(max_count),
-                       keys.cu_keys_dev.data_ptr() if keys is not None else None, mk,
-                       int(keys.max_keys) if keys is not None else int(max_count),
-                       float(scale), float(softcap), int(window), out.data_ptr(), ws.data_ptr(), self._stream())
+                       m, H, KV, cu_rows.data_ptr(), n_seq, int(max_count), ptr(new_len), ptr(table), table_w,
+                       ptr(k_pool), ptr(v_pool), page, rows_cap,
+                       float(scale), float(softcap), int(window), out.data_ptr(), int(shape), self._stream())
             return out
-        if keys is not None and (row_seq is None or row_pos is None):
-            raise KernelError("attention_prefill: gathered keys need every row's sequence and position")
+        if cached is not None and (row_seq is None or row_pos is None):
+            raise KernelError("attention_prefill: cached positions need every row's sequence and position")
         if row_seq is None:
             counts = (cu_rows[1:] - cu_rows[:-1]).long()
             row_seq = torch.repeat_interleave(torch.arange(n_seq, device=self.device, dtype=torch.int32), counts)
             row_pos = (torch.arange(m, device=self.device, dtype=torch.int32) - cu_rows[:-1][row_seq.long()]).to(torch.int32)
-        key_rows = cu_rows if keys is None else keys.key_row0_dev       # where a sequence's position 0 would lie
         self._call(self.lib, "tp_attn_simple_prefill", q.data_ptr(), qs, k.data_ptr(), ks, v.data_ptr(), vs, _code(q.dtype),
-                   m, H, KV, hd, key_rows.data_ptr(), row_seq.data_ptr(), row_pos.data_ptr(), float(scale), float(softcap),
+                   m, H, KV, hd, cu_rows.data_ptr(), row_seq.data_ptr(), row_pos.data_ptr(), ptr(new_len), ptr(table), table_w,
+                   ptr(k_pool), ptr(v_pool), page, rows_cap, float(scale), float(softcap),
                    int(window), out.data_ptr(), self._stream())
         return out
 
@@ -414,7 +399,7 @@ class HipOps:
         want = -(-(1536 if pairs < 192 else 768) // pairs)
         return max(1, min(want, -(-keys // 64), 128))
 
-    def _decode_pools(self, what, dtype, n, KV, hd, new_len, table, k_pool, v_pool):
+    def _check_pools(self, what, dtype, n, KV, hd, new_len, table, k_pool, v_pool):
         if new_len.numel() != n or new_len.dtype != torch.int32:
             raise KernelError(f"{what}: one int32 length per sequence")
         if k_pool.dtype != dtype or k_pool.dim() != 4 or tuple(k_pool.shape[1:]) != (KV, k_pool.shape[2], hd) \
@@ -430,7 +415,7 @@ class HipOps:
         qs = self._rows(q, "attention q")
         if q.shape[1] != H * hd:
             raise KernelError("attention_decode: q must be [sequences, heads * head_dim]")
-        self._decode_pools("attention_decode", q.dtype, n, KV, hd, new_len, table, k_pool, v_pool)
+        self._check_pools("attention_decode", q.dtype, n, KV, hd, new_len, table, k_pool, v_pool)
         out = torch.empty((n, H * hd), dtype=out_dtype, device=self.device)
         page = k_pool.shape[2]
         if self._fast_attention(q.dtype, H, KV, hd) and page >= 16 and page & (page - 1) == 0:
@@ -478,7 +463,7 @@ class HipOps:
             n_slices, slice_stride, row_stride = 1, 0, self._rows(rows, "attention_decode_step qkv")
         if rotary_dim and (inv_freq is None or inv_freq.dtype != torch.float32 or inv_freq.numel() != rotary_dim // 2):
             raise KernelError(f"attention_decode_step: a rotation over {rotary_dim} needs float32 inv_freq [{rotary_dim // 2}]")
-        self._decode_pools("attention_decode_step", torch.bfloat16, n, KV, hd, new_len, table, k_pool, v_pool)
+        self._check_pools("attention_decode_step", torch.bfloat16, n, KV, hd, new_len, table, k_pool, v_pool)
         lib = self.attn_lib(hd)
         keys = int(max_keys) if max_keys else k_pool.shape[0] * k_pool.shape[2]
         nsplit = int(splits) if splits else self.decode_splits(n, KV, hd, keys)

@@ -14,8 +14,9 @@ reads another run's cache projects and rotates its queries only.  In a decode st
 rotation, cache write and attention are one kernel launch where the kernel library
 has one for the geometry (`ops.fuses_decode_step`); the order of the arithmetic is
 the same.  A step that continues sequences by several tokens, or mixes starting and running sequences, attends
-over the cached positions its queries still see plus its own rows (the reference's multi-token step does the
-same from any position: runtime/src/lib.rs:676-720, runtime/cuda/codebook_gemv.cu:410-440).
+over the cached positions its queries still see, read in place through the page table, plus its own rows (the
+reference's multi-token step walks its cache from any position: runtime/src/lib.rs:676-720,
+runtime/cuda/codebook_gemv.cu:410-440), and caches its own rows after the attention.
 """
 from ..cache.store import KVSpec
 from ..models.spec import TensorSpec
@@ -77,32 +78,32 @@ class Attention(Mixer):
             q, k, v = qkv[:, :Q], qkv[:, Q:Q + KVD], qkv[:, Q + KVD:]
         else:
             q, k, v = ops.linear(x, self.w_qkv[:Q], ctx.dtype), None, None
-        keys = gathered = None
-        if ctx.mode == "extend":
-            # Sequences go on by several tokens (or some start while others go on): the queries see cached positions
-            # and the step's own rows.  The cached ones are copied out first, because the step's rows may take their
-            # places in a window's ring; the step's rows join them in the same buffers as they are rotated.
-            keys = ctx.keys_of(site.group_index)
-            if owns_cache:
-                gk, gv = ops.gather_kv_prefix(table, site.k, site.v, rows_cap, ctx.cu_rows, keys)
-                gathered = (gk, gv, keys.key_row0_dev)
-        ops.rope_kv_write(q, k, v, H, KV, hd, self.inv_freq, self.position.rotary_dim,
-                          ctx.row_seq, ctx.row_pos, ctx.new_len, table, site.k, site.v, rows_cap, gathered=gathered,
-                          pairing=pairing)
         if ctx.mode == "decode":
+            ops.rope_kv_write(q, k, v, H, KV, hd, self.inv_freq, self.position.rotary_dim,
+                              ctx.row_seq, ctx.row_pos, ctx.new_len, table, site.k, site.v, rows_cap, pairing=pairing)
             out = ops.attention_decode(q, H, KV, hd, ctx.new_len, table, site.k, site.v, rows_cap,
                                        self.query_scale, self.softcap, self.window, ctx.dtype,
                                        max_keys=ctx.max_keys(site))
+            return ops.linear(out, self.w_o, ctx.dtype, defer=True)
+        # Sequences that go on by several tokens (or some start while others go on) see cached positions and the
+        # step's own rows.  The attention reads the cached ones where they lie, as earlier steps left them, and the
+        # step's rows from the step; only then are the step's rows cached: in a window's ring without a row to spare
+        # they take the places of positions that the step's earlier queries still see.
+        extend = ctx.mode == "extend"
+        ops.rope_kv_write(q, k, v, H, KV, hd, self.inv_freq, self.position.rotary_dim,
+                          ctx.row_seq, ctx.row_pos, ctx.new_len, table, site.k, site.v, rows_cap, pairing=pairing,
+                          write=not extend)
+        if owns_cache:
+            ctx.offer_step_kv(k, v)
         else:
-            if gathered is not None:
-                k, v = gathered[0], gathered[1]
-            if owns_cache:
-                ctx.offer_step_kv(k, v)
-            else:
-                k, v = ctx.step_kv_of(ctx.cache_owner)
-            out = ops.attention_prefill(q, k, v, H, KV, hd, ctx.cu_rows, ctx.max_count,
-                                        self.query_scale, self.softcap, self.window, ctx.dtype,
-                                        row_seq=ctx.row_seq, row_pos=ctx.row_pos, keys=keys)
+            k, v = ctx.step_kv_of(ctx.cache_owner)
+        out = ops.attention_prefill(q, k, v, H, KV, hd, ctx.cu_rows, ctx.max_count,
+                                    self.query_scale, self.softcap, self.window, ctx.dtype,
+                                    row_seq=ctx.row_seq, row_pos=ctx.row_pos,
+                                    cached=(ctx.new_len, table, site.k, site.v, rows_cap) if extend else None)
+        if extend and owns_cache:
+            row_seq, row_pos, new_len, k_pool, v_pool = ctx.row_seq, ctx.row_pos, ctx.new_len, site.k, site.v
+            ctx.after_readers(lambda: ops.kv_write(k, v, KV, hd, row_seq, row_pos, new_len, table, k_pool, v_pool, rows_cap))
         return ops.linear(out, self.w_o, ctx.dtype, defer=True)
 
 
