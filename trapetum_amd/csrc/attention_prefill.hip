@@ -22,8 +22,15 @@
 // element, 8 keys per lane) comes out of LDS through ds_read_b64_tr_b16, the transposing read of gfx950, so no
 // transposed copy of V is ever made.
 // K and V tiles travel global memory -> LDS directly (global_load_lds_dwordx4), each into a single buffer: the
-// next K tile is asked for when every wave has multiplied the current one, the next V tile when every wave has
-// used the current one, so that a load has half a round to land and a round costs two barriers.
+// next K tile is asked for when every wave has multiplied the current one (in the middle of the softmax), the
+// next V tile when every wave has used the current one, so that each load has about half a round to land and a
+// round costs two barriers.  The first tiles are asked for before the queries.
+//
+// Measured on MI355X, Gemma-2 2B sizes (8 heads, 4 kv heads of 256, cap 50): 8 x 7,900 tokens 2.2 ms a layer
+// (0.92 PFLOP/s; matrix pipes busy half the time, no LDS bank conflicts), 2,048 tokens 50 us.  What was tried and
+// changed nothing there: fragments three and four ahead instead of two, a second chain of score accumulation,
+// half or all of the queries in LDS, the block's upper waves running half a round behind the lower ones (slower:
+// the halves differ in length and every wave waits for the slowest at both barriers).
 #include "common.h"
 
 #ifndef TP_HD
@@ -60,6 +67,7 @@ constexpr int MERGE_LANE = DT * 16 + 4;       // floats a lane hands over: its p
 // At head size 256 the output (128 registers a lane) and the queries (64) leave too little room for fragments in
 // flight: the last QL of a wave's query fragments live in LDS (1 KB each, one 16-byte read per lane and round).
 constexpr int QL = HD > 128 ? 4 : 0, QR = KS16 - QL;
+constexpr int KD = 2, VD = 2;                 // fragments of K (with the query fragment from LDS) and of V asked for ahead of their product
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr float LAZY = 8.f;                   // the running maximum moves only when a score exceeds it by this much (log 2 units)
 
@@ -95,8 +103,10 @@ template <int CG, int KG> struct PrefillShape {
 };
 }  // namespace
 
+// Registers: up to 256 a lane at head size 256 (two waves a SIMD); smaller heads need fewer, and a block of four
+// waves then runs three to a SIMD (27B sizes, 2 x 7,900 tokens: 1.62 -> 1.42 ms; four to a SIMD spill and lose).
 template <int CG, int KG, bool PAGED>
-__global__ void __launch_bounds__(64 * CG * KG, 2)
+__global__ void __launch_bounds__(64 * CG * KG, (HD <= 128 && CG * KG == 4 ? 3 : 2))
 attn_prefill_k(PrefillArgs a) {
     extern __shared__ __attribute__((aligned(16))) unsigned char prefill_lds[];
     bf16_t* const Kbuf = reinterpret_cast<bf16_t*>(prefill_lds);                  // [KG] tiles
@@ -118,20 +128,6 @@ attn_prefill_k(PrefillArgs a) {
     const int qw0 = start + q0 + (cg & (PT - 1)) * 32;           // position of the wave's first query
     const int qpos = qw0 + col;
     const bool q_ok = qpos < L;
-
-    // ---- the wave's queries: B operand of the first product, in registers for the whole kernel -----------------
-    // (the last QL of them in LDS, written by the column group's wave of key group 0)
-    pf_bf16x8 qf[QR];
-    uint4* const Qs = Qbuf + (cg * QL) * 64 + lane;
-    {
-        const bf16_t* qrow = a.q + (size_t)(row0 + (q_ok ? qpos : L - 1) - start) * a.q_stride + (size_t)h * HD + hi * 8;
-#pragma unroll
-        for (int ks = 0; ks < QR; ks++) qf[ks] = *reinterpret_cast<const pf_bf16x8*>(qrow + ks * 16);
-        if (QL > 0 && kg == 0) {
-#pragma unroll
-            for (int ks = QR; ks < KS16; ks++) Qs[(ks - QR) * 64] = *reinterpret_cast<const uint4*>(qrow + ks * 16);
-        }
-    }
 
     // ---- the keys the block walks: tiles of 32 positions, aligned to multiples of 32 ---------------------------
     int k_lo = a.window > 0 ? max(0, start + q0 - a.window + 1) : 0;
@@ -230,28 +226,47 @@ attn_prefill_k(PrefillArgs a) {
     rows_of_round(0);
     issue_k();
     issue_v();
+    // ---- the wave's queries: B operand of the first product, in registers for the whole kernel -----------------
+    // (the last QL of them in LDS, written by the column group's wave of key group 0)
+    pf_bf16x8 qf[QR];
+    uint4* const Qs = Qbuf + (cg * QL) * 64 + lane;
+    {
+        const bf16_t* qrow = a.q + (size_t)(row0 + (q_ok ? qpos : L - 1) - start) * a.q_stride + (size_t)h * HD + hi * 8;
+#pragma unroll
+        for (int ks = 0; ks < QR; ks++) qf[ks] = *reinterpret_cast<const pf_bf16x8*>(qrow + ks * 16);
+        if (QL > 0 && kg == 0) {
+#pragma unroll
+            for (int ks = QR; ks < KS16; ks++) Qs[(ks - QR) * 64] = *reinterpret_cast<const uint4*>(qrow + ks * 16);
+        }
+    }
+
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
+    float sc[16];                                    // lane: query `col`, keys kt + 8 (j / 4) + 4 hi + j % 4; in units of log 2
     for (int r = 0; r < n_rounds; r++) {
         const int kt = k_lo + 32 * (r * KG + kg);
         // wave-uniform: some key of the tile is visible to some query of the wave
         const bool visible = kt < k_hi && kt <= qw0 + 31 && qw0 < L && (a.window <= 0 || kt + 31 > qw0 - a.window);
-        float sc[16];                                // lane: query `col`, keys kt + 8 (j / 4) + 4 hi + j % 4; in units of log 2
         if (visible) {
-            // two chains of accumulation where the registers allow it (the instruction wants two independent ones
-            // in flight; at head size 256 there is no room, and the SIMD's other wave fills in)
+            // two chains of accumulation where the registers allow it (at head size 256 they do not, and a second
+            // chain measured no faster there: the SIMD's other wave fills in)
             constexpr bool TWO = KS16 > 1 && HD <= 128;
             pf_f32x16 s, s1;
 #pragma unroll
             for (int e = 0; e < 16; e++) { s[e] = 0.f; s1[e] = 0.f; }
+            PFrag kq[KD], qq[KD];                   // the fragments of k step ks in slot ks % KD
+            auto k_frag = [&](int ks) {
+                kq[ks % KD].u = *reinterpret_cast<const uint4*>(Kt + (ks >> 2) * (32 * 64) + koff[ks & 3]);
+                if (ks >= QR) qq[ks % KD].u = Qs[(ks - QR) * 64];
+            };
+#pragma unroll
+            for (int ks = 0; ks < KD - 1 && ks < KS16; ks++) k_frag(ks);
 #pragma unroll
             for (int ks = 0; ks < KS16; ks++) {
-                PFrag kf, qq;
-                kf.u = *reinterpret_cast<const uint4*>(Kt + (ks >> 2) * (32 * 64) + koff[ks & 3]);
-                if (ks < QR) qq.v = qf[ks < QR ? ks : 0];
-                else qq.u = Qs[(ks - QR) * 64];
-                if (TWO && (ks & 1)) s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf.v, qq.v, s1, 0, 0, 0);
-                else s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf.v, qq.v, s, 0, 0, 0);
+                if (ks + KD - 1 < KS16) k_frag(ks + KD - 1);
+                const pf_bf16x8 kf = kq[ks % KD].v, qv = ks < QR ? qf[ks < QR ? ks : 0] : qq[ks % KD].v;
+                if (TWO && (ks & 1)) s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qv, s1, 0, 0, 0);
+                else s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qv, s, 0, 0, 0);
             }
             if (TWO) s = s + s1;
             if (a.cap > 0.f) {                       // cap * tanh(x) = cap - 2 cap / (1 + e^(2x))
@@ -263,9 +278,10 @@ attn_prefill_k(PrefillArgs a) {
                 for (int j = 0; j < 16; j++) sc[j] = s[j] * scale2;
             }
         }
-        // (the barrier stands in the middle of the softmax so that both loads have about half a round to land)
-        __builtin_amdgcn_s_waitcnt(0);               // this round's V has landed, and
-        __syncthreads();                             // every wave has read the K tile: the next one may come
+        // The barrier stands in the middle of the softmax, so that both loads have about half a round to land: here
+        // this round's V tile has landed and every wave has read the K tile, whose successor may come.
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
         if (r + 1 < n_rounds) {
             rows_of_round(r + 1);
             issue_k();
@@ -320,16 +336,18 @@ attn_prefill_k(PrefillArgs a) {
                 }
                 return vf;
             };
-            PFrag vnext = v_frag(0);
+            PFrag vq[VD];
+#pragma unroll
+            for (int i = 0; i < VD - 1 && i < 2 * DT; i++) vq[i % VD] = v_frag(i);
 #pragma unroll
             for (int i = 0; i < 2 * DT; i++) {
-                const PFrag vf = vnext;
-                if (i + 1 < 2 * DT) vnext = v_frag(i + 1);
-                o[i % DT] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf.v, pf[i / DT].v, o[i % DT], 0, 0, 0);
+                if (i + VD - 1 < 2 * DT) vq[(i + VD - 1) % VD] = v_frag(i + VD - 1);
+                o[i % DT] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vq[i % VD].v, pf[i / DT].v, o[i % DT], 0, 0, 0);
             }
         }
-        __builtin_amdgcn_s_waitcnt(0);               // the next K tile has landed, and
-        __syncthreads();                             // every wave has used the V tile: the next one may come
+        // the next K tile has landed, and every wave has used the V tile, whose successor may come
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
         if (r + 1 < n_rounds) issue_v();
     }
 
@@ -450,15 +468,21 @@ extern "C" int tp_attn_prefill(const void* q, long q_stride, const void* k, long
         pt_shift = 0;
         while (((1 << gs) << (pt_shift + 1)) <= cg) pt_shift++;
     };
-    // Blocks of 4 column groups (two to a CU) where they give every CU at least two blocks; else 2 column groups
-    // and 4 key groups, so that a step of few query tiles still fills the chip and its longest chain of rounds is
-    // a quarter as long.
+    // Blocks of 4 column groups share a staged tile among the most queries and run two (three) to a CU out of step
+    // with one another: the choice where a step gives every CU four of them.  A smaller step gets its parallelism
+    // from the keys: 2 column groups x 2 key groups, or, for sequences of a thousand tokens and more where even those
+    // blocks are at most two a CU (at head sizes whose tiles let one 8-wave block fit a CU), 2 x 4: a quarter of the
+    // rounds for the longest block.  Measured for 4x1 / 2x2 / 2x4: 2B sizes, 2,048 tokens 94 / 61 / 51 us, 4,096 tokens
+    // 186 / 130 / 114, 8 x 512 tokens 34 / 27 / 36; 9B sizes, 2,048 tokens 100 / 72 / 69; 27B (heads of 128) 85 / 78 / 89.
     int cg = 4, kg = 1;
     {
         int gs, pts;
         plan(4, gs, pts);
         const long blocks4 = (long)tp_cdiv(max_count, 32 << pts) * n_seq * KV * (G >> gs);
-        if (shape == 2 || (shape == 0 && blocks4 < 2L * cus)) { cg = 2; kg = 4; }
+        plan(2, gs, pts);
+        const long blocks2 = (long)tp_cdiv(max_count, 32 << pts) * n_seq * KV * (G >> gs);
+        if (shape == 0 && blocks4 < 4L * cus) shape = HD > 128 && blocks2 <= 2L * cus && max_count >= 1024 ? 2 : 3;
+        if (shape == 2) { cg = 2; kg = 4; }
         if (shape == 3) { cg = 2; kg = 2; }
     }
     plan(cg, a.ghb_shift, a.pt_shift);
