@@ -185,7 +185,8 @@ def test_layer_0_is_local_and_layer_types_overrides(tmp_path, dtype):
 def test_no_layers_oracle_and_sandwich_identity(tmp_path, dtype):
     """Without layers the logits are norm(E[tok] * sqrt(D)) @ E^T (the lookup is scaled, the head is not), and with
     post-norm weights of -1 (a gain of 0) every layer adds nothing, so the same holds with layers.  Fails when a
-    post-norm is applied to the sub-layer's input instead of its output, or the head uses the scaled table."""
+    post-norm is applied after the residual sum instead of before it, or the head uses the scaled table.  (That the
+    post-norm takes the sub-layer's output, not its input, is what test_post_norms_stand_on_the_sub_layers_outputs pins.)"""
     import math
     folder = make_folder(tmp_path, "B", name="no_layers", num_hidden_layers=0)
     model, cfg = _model_of(folder, dtype)
@@ -212,3 +213,28 @@ def test_no_layers_oracle_and_sandwich_identity(tmp_path, dtype):
     assert rel_l2(_whole(model, toks), n @ e.T) < TOL[dtype]
     model, cfg = _model_of(folder, dtype)
     assert rel_l2(_whole(model, toks), n @ e.T) > 10 * TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_post_norms_stand_on_the_sub_layers_outputs(tmp_path, dtype):
+    """Output projections eight times as large leave the logits where they were, because the norm that follows a
+    sub-layer normalises that sub-layer's output before the residual sum (runtime/src/lib.rs:4530-4533) and an RMS norm
+    forgets its input's scale (up to eps).  With the post-norm on the sub-layer's input instead, the factor of eight
+    would reach the stream (the plain implementation's test of the same name shows that mistake moving the logits by more
+    than a tenth).  A factor of 8 is exact in bfloat16, so both engines see the same change."""
+    from trapetum_amd.weights import WeightFolder
+    folder = make_folder(tmp_path, "B")
+    src = WeightFolder(folder)
+    tensors = {name: src.tensor(name).clone() for name in src.names()}
+    src.close()
+    toks = random_tokens(19, 512, 2)
+    model, cfg = _model_of(folder, dtype, tensors)
+    ref = _whole(model, toks)
+    for name in tensors:
+        if name.endswith("self_attn.o_proj.weight") or name.endswith("mlp.down_proj.weight"):
+            tensors[name] = tensors[name] * 8.0
+    model, cfg = _model_of(folder, dtype, tensors)
+    got = _whole(model, toks)
+    assert rel_l2(got, ref) < (1e-3 if dtype == "float32" else 2e-2), rel_l2(got, ref)
+    pcfg, pw = plain.read_folder(folder)
+    assert rel_l2(got, plain.forward(pcfg, pw, toks)) < 2 * TOL[dtype] + 1e-3

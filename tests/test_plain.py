@@ -7,7 +7,7 @@ import pytest
 import torch
 
 from .plain import gemma2_plain as plain
-from .tiny import TINY_A, TINY_B, make_folder, random_tokens
+from .tiny import TINY_A, TINY_B, make_folder, random_tokens, rel_l2
 
 D = torch.float64
 
@@ -164,6 +164,34 @@ def test_no_layers_oracle_and_sandwich_identity(folder_b):
     capped = plain.forward(dict(cfg, final_logit_softcapping=3.0), w, toks)
     assert float(capped.abs().max()) <= 3.0
     assert torch.equal(capped.argmax(-1), plain.forward(cfg, w, toks).argmax(-1))           # the cap is monotone
+
+
+def test_post_norms_stand_on_the_sub_layers_outputs(folder_b):
+    """The norm after the mixer (and after the feed-forward) normalises that sub-layer's OUTPUT before the residual sum
+    (runtime/src/lib.rs:4530-4533): an RMS norm forgets its input's scale, so output projections eight times as large
+    leave the logits where they were (up to the norm's eps).  A post-norm applied to the sub-layer's input instead, or
+    none at all, lets the factor of eight through."""
+    cfg, w = plain.read_folder(folder_b)
+    toks = random_tokens(19, cfg["vocab_size"], 2)
+    w8 = dict(w)
+    for l in range(cfg["num_hidden_layers"]):
+        for name in ("self_attn.o_proj", "mlp.down_proj"):
+            w8[f"model.layers.{l}.{name}.weight"] = 8.0 * w[f"model.layers.{l}.{name}.weight"]
+    ref, got = plain.forward(cfg, w, toks), plain.forward(cfg, w8, toks)
+    assert rel_l2(got, ref) < 1e-3, rel_l2(got, ref)
+
+    def post_norm_on_the_input(x, positions, W, layer, c, rnd):     # the mistake: it passes the factor on
+        p = f"model.layers.{layer}."
+        n = plain.rms_norm(plain.rms_norm(x, W[p + "input_layernorm.weight"], c["rms_norm_eps"]), W[p + "post_attention_layernorm.weight"], c["rms_norm_eps"])
+        x = x + plain.attention_block(n, positions, W, p, c, plain.layer_window(c, layer), rnd)
+        n = plain.rms_norm(plain.rms_norm(x, W[p + "pre_feedforward_layernorm.weight"], c["rms_norm_eps"]), W[p + "post_feedforward_layernorm.weight"], c["rms_norm_eps"])
+        return x + plain.geglu(n, W[p + "mlp.gate_proj.weight"], W[p + "mlp.up_proj.weight"], W[p + "mlp.down_proj.weight"], rnd)
+    right = plain.block
+    try:
+        plain.block = post_norm_on_the_input
+        assert rel_l2(plain.forward(cfg, w8, toks), plain.forward(cfg, w, toks)) > 0.1
+    finally:
+        plain.block = right
 
 
 def test_shifting_all_positions_changes_nothing(folder_b):

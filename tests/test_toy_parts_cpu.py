@@ -1,4 +1,4 @@
-"""A toy mixer with a state of its own, another position table, a feed-forward with a router over experts and a
+"""A toy mixer with a state of its own, one that keeps a single tensor per token in a window's ring, another position table, a feed-forward with a router over experts and a
 schedule that runs a layer twice and shares a cache: registered, built and stepped without a change to the framework
 (host logic, CPU)."""
 import pytest
@@ -32,9 +32,17 @@ def toy(tmp_path_factory):
 def test_cache_groups_of_the_toy(toy):
     model, _ = toy
     cache = model.new_cache(max_tokens=256, page_size=16)
-    assert len(cache.kv_groups) == 1 and cache.kv_groups[0].entries == [1]          # entry 3 reads entry 1's cache
-    assert len(cache.state_groups) == 1 and cache.state_groups[0].entries == [0, 2]  # layer 0 runs twice: two states
-    assert cache.site(3) is None
+    attn, mem = cache.token_groups
+    assert attn.entries == [1] and sorted(attn.pools) == ["k", "v"]                  # entry 4 reads entry 1's cache
+    # the mixer that keeps one tensor per token has one pool, a ring of its window: nothing else is allocated for it
+    assert mem.entries == [2] and list(mem.pools) == ["h"] and mem.pages.rows_cap == 16
+    assert tuple(mem.pools["h"].shape) == (1, 16 + 1, 16, toy_parts.TOY["mem"])
+    assert cache.bytes() == sum(p.numel() * p.element_size() for g in cache.token_groups for p in g.pools.values()) + \
+        sum(g.tensor.numel() * g.tensor.element_size() for g in cache.state_groups)
+    assert len(cache.state_groups) == 1 and cache.state_groups[0].entries == [0, 3]  # layer 0 runs twice: two states
+    assert cache.site(4) is None
+    with pytest.raises(Exception, match="keeps no per-token tensor 'v'"):
+        cache.site(2).tensor("v")
 
 
 def test_toy_whole_stepwise_and_batched(toy):

@@ -16,6 +16,8 @@ def _lib():
     lib.tp_last_error.restype = ctypes.c_char_p
     lib.tp_argmax_no_alloc.argtypes = [P, I, I, P, P]
     lib.tp_argmax_no_alloc.restype = I
+    lib.tp_argmax_no_alloc_prepare.argtypes = []
+    lib.tp_argmax_no_alloc_prepare.restype = I
     lib.tp_argmax.argtypes = [P, I, I, P, P, P]
     lib.tp_argmax.restype = I
     lib.tp_argmax_workspace_bytes.argtypes = [I, I]
@@ -50,3 +52,40 @@ def test_no_alloc_argmax_refuses_what_the_scratch_cannot_hold():
     assert lib.tp_argmax_no_alloc(z.data_ptr(), 257, 8, out.data_ptr(), None) != 0
     assert b"256" in lib.tp_last_error()
     assert lib.tp_argmax_no_alloc(z.data_ptr(), 0, 8, out.data_ptr(), None) != 0
+
+
+def test_no_alloc_argmax_inside_a_captured_graph():
+    """What the header names as a caller: after tp_argmax_no_alloc_prepare() (outside the capture) two calls, a large one
+    and then a smaller one, are captured into one HIP graph; every replay, with other work and synchronisations of the
+    program between the replays and new logits each time, gives what tp_argmax gives."""
+    lib = _lib()
+    dev = torch.device("cuda:0")
+    assert lib.tp_argmax_no_alloc_prepare() == 0, lib.tp_last_error()
+    shapes = ((8, 256000), (3, 50021))
+    z = [torch.zeros(s, device=dev) for s in shapes]
+    got = [torch.full((s[0],), -1, dtype=torch.int32, device=dev) for s in shapes]
+    side = torch.cuda.Stream(device=dev)
+    side.wait_stream(torch.cuda.current_stream(dev))
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            st = torch.cuda.current_stream(dev).cuda_stream
+            for t, o in zip(z, got):
+                assert lib.tp_argmax_no_alloc(t.data_ptr(), t.shape[0], t.shape[1], o.data_ptr(), st) == 0, lib.tp_last_error()
+    torch.cuda.current_stream(dev).wait_stream(side)
+    g = torch.Generator().manual_seed(12)
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    for replay in range(4):
+        for t in z:
+            t.copy_(torch.randn(t.shape, generator=g))
+            t[1, (replay * 7919) % t.shape[1]] = 9.0
+        graph.replay()
+        torch.cuda.synchronize(dev)
+        for t, o in zip(z, got):
+            want = torch.empty(t.shape[0], dtype=torch.int32, device=dev)
+            ws = torch.empty(lib.tp_argmax_workspace_bytes(*t.shape), dtype=torch.uint8, device=dev)
+            assert lib.tp_argmax(t.data_ptr(), t.shape[0], t.shape[1], want.data_ptr(), ws.data_ptr(), stream) == 0
+            torch.cuda.synchronize(dev)
+            assert o.tolist() == want.tolist(), replay
+            assert o.tolist()[1] == (replay * 7919) % t.shape[1]
+            o.fill_(-1)

@@ -1,5 +1,5 @@
 """Toy parts defined by the tests, registered from outside the framework: a mixer with a state of fixed size
-per sequence, another position table, a feed-forward with a router over experts, a norm of another kind, and an
+per sequence, a mixer that keeps one tensor per token (in a window's ring), another position table, a feed-forward with a router over experts, a norm of another kind, and an
 architecture that mixes them with the built-in parts (one layer has two kinds of norm and a SiLU-gated feed-forward).  They are no model of anyone's; they show that the framework's files need no change
 for a new part."""
 import dataclasses
@@ -7,7 +7,7 @@ import math
 
 import torch
 
-from trapetum_amd.cache import StateSpec
+from trapetum_amd.cache import StateSpec, TokenSpec
 from trapetum_amd.config.base import ModelConfig, key
 from trapetum_amd.models.spec import LayerSpec, ModelSpec, ScheduleEntry, TensorSpec
 from trapetum_amd.parts import FeedForward, Mixer, Norm, Position
@@ -45,6 +45,49 @@ class EmaMixer(Mixer):
             state[slot] = s
             row += count
         return ctx.ops.linear(out.to(ctx.dtype), self.w, ctx.dtype, bias=self.b)       # a projection with a bias
+
+
+class WindowMeanMixer(Mixer):
+    """Keeps ONE tensor per token, h_t = in_proj(x_t) of `mem` elements, for the last `window` tokens;
+    out_t = out_proj(mean of h_s over the tokens s <= t with t - s < window).  It reads what earlier steps cached
+    through the page table (a ring's rows where the window is shorter than the context), then caches its own rows."""
+
+    def __init__(self, hidden_size, mem, window):
+        self.hidden_size, self.mem, self.window = hidden_size, mem, int(window)
+
+    def tensor_specs(self):
+        return {"in_proj.weight": TensorSpec((self.mem, self.hidden_size)), "out_proj.weight": TensorSpec((self.hidden_size, self.mem))}
+
+    def cache_spec(self):
+        return TokenSpec.of(self.window, h=(self.mem,))
+
+    def bind(self, tensors, rt):
+        self.rt = rt
+        self.w_in, self.w_out = rt.matrix(tensors["in_proj.weight"]), rt.matrix(tensors["out_proj.weight"])
+
+    def forward(self, ctx, x, site):
+        pool = site.tensor("h")                              # [pages, page, mem]
+        table = ctx.page_table(site.group_index).long()
+        page, cap, W = pool.shape[1], site.rows_cap, self.window
+        h = ctx.ops.linear(x, self.w_in, ctx.dtype)
+        out = torch.empty((x.shape[0], self.mem), dtype=torch.float32, device=x.device)
+        row = 0
+        for i, (start, count) in enumerate(zip(ctx.starts, ctx.counts)):
+            lo = max(0, start - (W - 1))
+            pos = torch.arange(lo, start, device=x.device)
+            rows = pos % cap if cap else pos
+            seen = torch.cat([pool[table[i][rows // page], rows % page], h[row:row + count]]).float()     # positions lo ..
+            for r in range(count):
+                p = start + r
+                out[row + r] = seen[max(lo, p - W + 1) - lo:p - lo + 1].mean(0)
+            for r in range(count):                           # the step's own rows, cached after they were read
+                p = start + r
+                if cap and p + cap < start + count:
+                    continue                                 # a later row of this step lands on the same ring row
+                rr = p % cap if cap else p
+                pool[table[i][rr // page], rr % page] = h[row + r]
+            row += count
+        return ctx.ops.linear(out.to(ctx.dtype), self.w_out, ctx.dtype)
 
 
 class SoftRoutedMLP(FeedForward):
@@ -125,6 +168,8 @@ class ToyConfig(ModelConfig):
     decay: float = key("decay", "float")
     rotary: int = key("rotary", "int")
     experts: int = key("experts", "int")
+    mem: int = key("mem", "int")
+    mem_window: int = key("mem_window", "int")
 
 
 def toy_spec(c):
@@ -132,14 +177,18 @@ def toy_spec(c):
     layers = []
     for l in range(c.n_layers):
         p = f"blocks.{l}."
-        if l % 2 == 0:
+        if l == 2:
+            mixer = ("toy_window_mean", {"hidden_size": c.width, "mem": c.mem, "window": c.mem_window})
+        elif l % 2 == 0:
             mixer = ("toy_ema", {"hidden_size": c.width, "decay": c.decay})
         else:
             mixer = ("attention", {"hidden_size": c.width, "num_heads": c.heads, "num_kv_heads": c.heads,
                                    "head_dim": c.head_size, "query_scale": 1.0 / math.sqrt(c.head_size),
                                    "position": ("toy_squared", {"rotary_dim": c.rotary})})
         norms = None
-        if l % 2 == 0:      # a SiLU gate, and a second kind of norm in front of it
+        if l == 2:
+            ff = ("gated_mlp", {"hidden_size": c.width, "intermediate_size": c.ff_width, "activation": "gelu_tanh"})
+        elif l % 2 == 0:    # a SiLU gate, and a second kind of norm in front of it
             ff = ("gated_mlp", {"hidden_size": c.width, "intermediate_size": c.ff_width, "activation": "silu"})
             norms = {"pre_ff_norm": ("toy_centered_norm", {"size": c.width, "eps": c.eps})}
         else:
@@ -159,13 +208,15 @@ def toy_spec(c):
 
 def register():
     register_part("mixer", "toy_ema", EmaMixer)
+    register_part("mixer", "toy_window_mean", WindowMeanMixer)
     register_part("position", "toy_squared", SquaredPosition)
     register_part("norm", "toy_centered_norm", CenteredNorm)
     register_part("feed_forward", "toy_soft_routed", SoftRoutedMLP)
     register_architecture(ToyConfig.architecture, ToyConfig, toy_spec)
 
 
-TOY = dict(n_layers=2, width=48, heads=3, head_size=16, ff_width=80, vocab=97, eps=1e-5, decay=0.8, rotary=8, experts=3)
+TOY = dict(n_layers=3, width=48, heads=3, head_size=16, ff_width=80, vocab=97, eps=1e-5, decay=0.8, rotary=8, experts=3,
+           mem=24, mem_window=11)
 
 
 # ---- the toy's own plain reference: whole sequences, float64, no cache ------------------------------------------------
@@ -209,12 +260,19 @@ def toy_reference(cfg, W, tokens):
         o = torch.einsum("hts,shd->thd", torch.softmax(sc, -1), v).reshape(T, H * hd)
         return o @ W[p + "mix.o_proj.weight"].T, kv
 
+    def window_mean(t, p):
+        h = t @ W[p + "mix.in_proj.weight"].T
+        m = torch.stack([h[max(0, r - cfg["mem_window"] + 1):r + 1].mean(0) for r in range(T)])
+        return m @ W[p + "mix.out_proj.weight"].T
+
     kv1 = None
-    for l, reuse in [(0, False), (1, False), (0, False), (1, True)]:
+    for l, reuse in [(0, False), (1, False), (2, False), (0, False), (1, True)]:
         p = f"blocks.{l}."
         n = norm(x, W[p + "n1.weight"])
         if l == 0:
             x = x + ema(n, p)
+        elif l == 2:
+            x = x + window_mean(n, p)
         else:
             a, kv = attn(n, p, kv1 if reuse else None)
             kv1 = kv1 or kv
@@ -229,6 +287,8 @@ def toy_reference(cfg, W, tokens):
             return (act(t @ W[q + "gate_proj.weight"].T) * (t @ W[q + "up_proj.weight"].T)) @ W[q + "down_proj.weight"].T
         if l == 0:
             x = x + mlp(n, p + "ff.", lambda g: g * torch.sigmoid(g))
+        elif l == 2:
+            x = x + mlp(n, p + "ff.")
         else:
             mix = torch.softmax(n @ W[p + "ff.router.weight"].T, -1)
             x = x + sum(mix[:, e:e + 1] * mlp(n, p + f"ff.experts.{e}.") for e in range(cfg["experts"]))

@@ -1,2 +1,2 @@
 from .slots import CacheError, FreeList, GroupPages, SlotBook   # noqa: F401
-from .store import CacheSite, KVSpec, ModelCache, StateSpec   # noqa: F401
+from .store import CacheSite, ModelCache, StateSpec, TokenSpec   # noqa: F401

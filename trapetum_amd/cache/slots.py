@@ -1,6 +1,6 @@
 """Book-keeping of the cache on the host: slots, pages, lengths.
 
-A slot stands for one live sequence.  Keys and values live in pages of
+A slot stands for one live sequence.  What is kept per token lives in pages of
 `page_size` rows drawn from one pool per group of layers; a slot's page list in
 a group grows as its sequence grows and goes back to the pool when the slot is
 released.  The reference keeps one dense buffer of max_seq rows per layer for

@@ -1,12 +1,17 @@
 """The cache's device storage.
 
 Every run of a layer (a schedule entry) that keeps something between steps
-declares what: keys and values (all of them, or a window), or a state of fixed
-size.  Entries with the same needs form a group with storage of its own:
+declares what: tensors per token (of all tokens, or of a window of them), or a
+state of fixed size.  Entries with the same needs form a group with storage of
+its own:
 
-  keys/values  pools  K, V [entries, pages, kv_heads, page_size, head_dim]; a
-               sequence's rows are found through its page list.  A window group
-               keeps a ring: position p lives in ring row p % rows_cap.
+  per token    one pool per named tensor; a tensor of shape (*lead, d) per token
+               lives in a pool [entries, pages, *lead, page_size, d] (a page's rows
+               stand before the last dimension, so that a row of d elements is
+               contiguous); a sequence's rows are found through its page list.  A
+               window group keeps a ring: position p lives in ring row p % rows_cap.
+               (Attention declares keys and values, each (kv_heads, head_dim); a
+               mixer that keeps one tensor per token declares one.)
   state        [entries, slots, *shape], zeroed when a slot is taken.
 
 Beyond what sequences can take, every pool has one spare page and every state one
@@ -27,10 +32,24 @@ from .slots import CacheError, GroupPages, SlotBook
 
 
 @dataclasses.dataclass(frozen=True)
-class KVSpec:
-    kv_heads: int
-    head_dim: int
-    window: Optional[int] = None        # None: every key is kept
+class TokenSpec:
+    """What a mixer keeps of every token: named tensors, each of a fixed shape, in the engine's activation dtype."""
+    tensors: tuple                      # ((name, shape), ...): hashable, in the mixer's order
+    window: Optional[int] = None        # None: every token is kept
+
+    @staticmethod
+    def of(window=None, **tensors):
+        """TokenSpec.of(window, k=(kv_heads, head_dim), v=(kv_heads, head_dim))"""
+        for name, shape in tensors.items():
+            if not shape or any(int(n) <= 0 for n in shape):
+                raise CacheError(f"per-token tensor '{name}' needs a shape of positive sizes, found {shape!r}")
+        return TokenSpec(tuple((name, tuple(int(n) for n in shape)) for name, shape in tensors.items()), window)
+
+    def shape_of(self, name):
+        for n, shape in self.tensors:
+            if n == name:
+                return shape
+        raise CacheError(f"the cache keeps no per-token tensor '{name}' here (it keeps {[n for n, _ in self.tensors]})")
 
 
 @dataclasses.dataclass(frozen=True)
@@ -49,16 +68,13 @@ class CacheSite:
         self._group = group
 
     @property
-    def is_kv(self):
-        return isinstance(self.spec, KVSpec)
+    def per_token(self):
+        return isinstance(self.spec, TokenSpec)
 
-    @property
-    def k(self):
-        return self._group.k_pool[self.index_in_group]
-
-    @property
-    def v(self):
-        return self._group.v_pool[self.index_in_group]
+    def tensor(self, name):
+        """The pool of one of the per-token tensors the entry declared: [pages, *lead, page_size, d]."""
+        self.spec.shape_of(name)
+        return self._group.pools[name][self.index_in_group]
 
     @property
     def rows_cap(self):
@@ -69,7 +85,7 @@ class CacheSite:
         return self._group.tensor[self.index_in_group]
 
 
-class _KVGroup:
+class _TokenGroup:
     def __init__(self, spec, entries, n_pages, max_slots, page_size, max_context, dtype, device, name):
         self.spec = spec
         self.entries = entries
@@ -79,9 +95,9 @@ class _KVGroup:
             n_pages = min(n_pages, max_slots * (rows_cap // page_size))      # a ring never grows beyond its rows
         self.pages = GroupPages(n_pages, page_size, rows_cap, name)
         self.spare_page = n_pages                                          # the pool's last page, never handed out
-        shape = (len(entries), n_pages + 1, spec.kv_heads, page_size, spec.head_dim)
-        self.k_pool = torch.zeros(shape, dtype=dtype, device=device)
-        self.v_pool = torch.zeros(shape, dtype=dtype, device=device)
+        self.pools = {}
+        for tname, shape in spec.tensors:
+            self.pools[tname] = torch.zeros((len(entries), n_pages + 1) + shape[:-1] + (page_size, shape[-1]), dtype=dtype, device=device)
         self.max_pages_per_seq = self.pages.max_pages(max_context)
 
 
@@ -96,7 +112,7 @@ class _StateGroup:
 class ModelCache:
     """Slots, pages and storage for one model instance.
 
-    entry_specs: for every schedule entry a KVSpec, a StateSpec or None.
+    entry_specs: for every schedule entry a TokenSpec, a StateSpec or None.
     max_tokens:  tokens that live sequences may hold together, each rounded up to a page.
     max_context: longest single sequence.
     """
@@ -110,18 +126,18 @@ class ModelCache:
         self.max_slots = max_slots
         self.spare_slot = max_slots           # a slot no sequence takes: see the module's text
         n_pages = max(1, -(-max_tokens // page_size))
-        self.kv_groups, self.state_groups = [], []
+        self.token_groups, self.state_groups = [], []
         self._site_of = {}
         keyed = {}
         for entry, spec in enumerate(entry_specs):
             if spec is not None:
                 keyed.setdefault(spec, []).append(entry)
         for spec, entries in keyed.items():
-            if isinstance(spec, KVSpec):
-                name = f"kv{len(self.kv_groups)}:" + ("all" if spec.window is None else f"window{spec.window}")
-                g = _KVGroup(spec, entries, n_pages, max_slots, page_size, max_context, dtype, device, name)
-                gi = len(self.kv_groups)
-                self.kv_groups.append(g)
+            if isinstance(spec, TokenSpec):
+                name = f"tokens{len(self.token_groups)}:" + ("all" if spec.window is None else f"window{spec.window}")
+                g = _TokenGroup(spec, entries, n_pages, max_slots, page_size, max_context, dtype, device, name)
+                gi = len(self.token_groups)
+                self.token_groups.append(g)
             elif isinstance(spec, StateSpec):
                 g = _StateGroup(spec, entries, max_slots, dtype, device)
                 gi = len(self.state_groups)
@@ -130,7 +146,7 @@ class ModelCache:
                 raise CacheError(f"schedule entry declares an unknown cache need: {spec!r}")
             for i, entry in enumerate(entries):
                 self._site_of[entry] = CacheSite(spec, gi, i, g)
-        self.book = SlotBook(max_slots, [g.pages for g in self.kv_groups], max_context)
+        self.book = SlotBook(max_slots, [g.pages for g in self.token_groups], max_context)
 
     # --- what parts use -------------------------------------------------------------
     def site(self, entry):
@@ -164,7 +180,7 @@ class ModelCache:
     def page_table(self, group_index, slots, width=None):
         """int32 [len(slots), width]: page ids of each slot in a group, -1 where it has none; the spare slot's row
         names the spare page."""
-        g = self.kv_groups[group_index]
+        g = self.token_groups[group_index]
         width = width or max(1, max(len(g.pages.lists.get(s, ())) for s in slots))
         t = np.full((len(slots), width), -1, dtype=np.int32)
         for i, s in enumerate(slots):
@@ -177,8 +193,8 @@ class ModelCache:
 
     def bytes(self):
         n = 0
-        for g in self.kv_groups:
-            n += 2 * g.k_pool.numel() * g.k_pool.element_size()
+        for g in self.token_groups:
+            n += sum(p.numel() * p.element_size() for p in g.pools.values())
         for g in self.state_groups:
             n += g.tensor.numel() * g.tensor.element_size()
         return n

@@ -20,7 +20,14 @@ extern "C" {
 // (non-zero return, text from tp_last_error()).  Enqueued on `stream` (a hipStream_t); calls no hipMalloc, hipFree or
 // allocating library routine.  Each GPU holds one scratch array of TP_ARGMAX_NO_ALLOC_SCRATCH_BYTES that every call
 // on that GPU shares: calls that overlap on one GPU race; calls in stream order do not.
+// The first call on a device also asks the runtime where that device's copy of the array lies, which is no stream
+// operation (it may load the library's code on that device): make that first call, or tp_argmax_no_alloc_prepare(),
+// outside any stream capture; every later call on the device only enqueues two kernels and may be captured.
 int tp_argmax_no_alloc(const float* logits, int B, int V, int* out, void* stream);
+
+// Resolves the scratch array's address on the current device and launches nothing: for callers that want the first
+// tp_argmax_no_alloc on a device to be inside a stream capture.  Returns 0, or non-zero with a message.
+int tp_argmax_no_alloc_prepare(void);
 
 #ifdef __cplusplus
 }

@@ -135,6 +135,11 @@ int scratch_address(void** out) {
 }
 }  // namespace
 
+extern "C" int tp_argmax_no_alloc_prepare(void) {
+    void* base = nullptr;
+    return scratch_address(&base);
+}
+
 extern "C" int tp_argmax_no_alloc(const float* logits, int B, int V, int* out, void* stream) {
     TP_REQUIRE(logits && out, "argmax_no_alloc: logits and output must be given");
     TP_REQUIRE(B > 0 && V > 0, "argmax_no_alloc: empty shape B=%d V=%d", B, V);

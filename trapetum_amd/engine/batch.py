@@ -43,7 +43,7 @@ def step_arrays(cache, slots, counts, starts, want_rows, table_widths=None):
         raise StepError(f"wanted rows {list(want_rows)} reach outside the step's {m} rows")
     parts = [np.asarray(slots), cu, row_seq, row_pos, new_len, want]
     shapes = []
-    for gi in range(len(cache.kv_groups)):
+    for gi in range(len(cache.token_groups)):
         t = cache.page_table(gi, slots, None if table_widths is None else table_widths[gi])
         shapes.append(t.shape)
         parts.append(t.reshape(-1))
@@ -62,7 +62,7 @@ class StaticStep:
         import torch
         self.rt = rt
         self.n_seq = n_seq
-        self.table_widths = [g.max_pages_per_seq for g in cache.kv_groups]
+        self.table_widths = [g.max_pages_per_seq for g in cache.token_groups]
         self.geometry = 6 * n_seq + 1 + sum(n_seq * w for w in self.table_widths)
         self.size = self.geometry + extra
         self.device_buffer = torch.zeros(self.size, dtype=torch.int32, device=rt.device)
@@ -112,8 +112,8 @@ class StepContext:
         self.cache_owner = None         # entry whose cache it uses
         self.static = static
         self.length_bound = length_bound
-        self._shared = set()            # entries whose step keys/values a later entry reads
-        self._step_kv = {}
+        self._shared = set()            # entries whose cache a later entry reads
+        self._step_rows = {}
         n, m = self.n_seq, self.n_rows
         self._after_step = []           # work put off until every entry of the step has run
         flat, shapes = step_arrays(cache, self.slots, self.counts, self.starts, want_rows,
@@ -153,25 +153,25 @@ class StepContext:
         print(f"[ldump] L={-1 if self.entry is None else self.entry} stage={stage} l2={float(t.norm()):.6e} "
               f"absmax={float(t.abs().max()):.6e} mean={float(t.mean()):.6e}", file=sys.stderr, flush=True)
 
-    def max_keys(self, site):
-        """Most keys any sequence of this step can see at this cache site (a host number, for launch geometry).
+    def max_rows_visible(self, site):
+        """Most cached rows any sequence of this step can see at this cache site (a host number, for launch geometry).
         With fixed step memory (a captured graph) it is the graph's bound on the lengths."""
         longest = max(s + c for s, c in zip(self.starts, self.counts))
         if self.length_bound is not None:
             longest = max(longest, self.length_bound)
         return min(longest, site.rows_cap) if site.rows_cap else longest
 
-    # keys and values of this step, for entries that read another entry's cache during a prefill
+    # what the running entry is about to cache of this step's rows, for the entries that read its cache in this step
     def mark_shared(self, entries):
         self._shared = set(entries)
 
-    def offer_step_kv(self, k, v):
-        """k, v: this step's own rows of the running entry, for the entries that read its cache."""
+    def offer_step_rows(self, **tensors):
+        """tensors: this step's own rows of the running entry's per-token tensors, by name."""
         if self.entry in self._shared:
-            self._step_kv[self.entry] = (k, v)
+            self._step_rows[self.entry] = tensors
 
-    def step_kv_of(self, entry):
-        return self._step_kv[entry]
+    def step_rows_of(self, entry):
+        return self._step_rows[entry]
 
     def after_readers(self, work):
         """Run `work()` once nobody in this step reads the running entry's cache as earlier steps left it any more:

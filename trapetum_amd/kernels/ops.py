@@ -98,7 +98,8 @@ class HipOps:
         plain = flags.force_plain()
         self.force_linear = 1 if plain else 0   # 1 plain, 2 skinny, 3 tiled (6: its wide tile, 7: its 128 x 96 tile, 8, 9: loads into LDS, 128 x 128 and 128 x 96), 4 multiply-adds (1-2 rows)
         self.force_plain_attention = plain
-        self._timed = None                      # with TRAPETUM_AMD_PROFILE=1: [(entry point, start event, end event)]
+        self._timed = None                      # with TRAPETUM_AMD_PROFILE=1: [(entry point, start event, end event)] not yet summed
+        self._profile_totals = {}               # entry point -> (milliseconds, calls)
         if flags.profile():
             import atexit
             self._timed = []
@@ -115,22 +116,34 @@ class HipOps:
             rc = getattr(lib, name)(*args)
             b.record()
             self._timed.append((name, a, b))
+            if len(self._timed) >= self.PROFILE_FOLD:
+                self._fold_profile()            # so that a long run holds a bounded number of events
         else:
             rc = getattr(lib, name)(*args)
         if rc != 0:
             raise KernelError(lib.tp_last_error().decode())
 
+    PROFILE_FOLD = 4096                         # timed calls kept as events before they are summed
+
+    def _fold_profile(self):
+        """Sum the timed calls so far into the totals per entry point and let go of their events."""
+        if not self._timed:
+            return
+        self._timed[-1][2].synchronize()
+        for name, a, b in self._timed:
+            ms, n = self._profile_totals.get(name, (0.0, 0))
+            self._profile_totals[name] = (ms + a.elapsed_time(b), n + 1)
+        self._timed = []
+
     def profile_report(self, file=None):
         """The time of the calls so far per entry point, most expensive first (TRAPETUM_AMD_PROFILE=1); forgets them."""
         import sys
-        if not self._timed:
+        if self._timed is None:
             return
-        torch.cuda.synchronize(self.device)
-        total = {}
-        for name, a, b in self._timed:
-            ms, n = total.get(name, (0.0, 0))
-            total[name] = (ms + a.elapsed_time(b), n + 1)
-        self._timed = []
+        self._fold_profile()
+        total, self._profile_totals = self._profile_totals, {}
+        if not total:
+            return
         out = file or sys.stderr
         for name, (ms, n) in sorted(total.items(), key=lambda kv: -kv[1][0]):
             print(f"[profile] op={name} calls={n} total_ms={ms:.3f} mean_us={1e3 * ms / n:.2f}", file=out, flush=True)

@@ -18,7 +18,7 @@ over the cached positions its queries still see, read in place through the page 
 reference's multi-token step walks its cache from any position: runtime/src/lib.rs:676-720,
 runtime/cuda/codebook_gemv.cu:410-440), and caches its own rows after the attention.
 """
-from ..cache.store import KVSpec
+from ..cache.store import TokenSpec
 from ..models.spec import TensorSpec
 from ..registry import build_part, register_part
 from .base import Mixer
@@ -46,7 +46,8 @@ class Attention(Mixer):
                 "v_proj.weight": TensorSpec((kv, d)), "o_proj.weight": TensorSpec((d, q))}
 
     def cache_spec(self):
-        return KVSpec(self.num_kv_heads, self.head_dim, self.window or None)
+        per_token = (self.num_kv_heads, self.head_dim)
+        return TokenSpec.of(self.window or None, k=per_token, v=per_token)
 
     def bind(self, tensors, rt):
         import torch
@@ -64,14 +65,15 @@ class Attention(Mixer):
         if site.spec.window is not None and not 0 < self.window <= site.spec.window:
             raise ValueError(f"this attention sees {self.window or 'all'} keys back, the cache it reads keeps {site.spec.window}")
         table = ctx.page_table(site.group_index)
+        k_pool, v_pool = site.tensor("k"), site.tensor("v")         # [pages, kv_heads, page, head_dim]
         rows_cap = site.rows_cap or 0
         pairing = self.position.pairing
-        if ctx.mode == "decode" and pairing == "halves" and ops.fuses_decode_step(ctx.dtype, H, KV, hd, site.k):
+        if ctx.mode == "decode" and pairing == "halves" and ops.fuses_decode_step(ctx.dtype, H, KV, hd, k_pool):
             # one launch rotates, writes the cache and attends; the projections may stay in K slices until then
             qkv = ops.linear(x, self.w_qkv if owns_cache else self.w_qkv[:Q], ctx.dtype, defer=True)
             out = ops.attention_decode_step(qkv, H, KV, hd, self.inv_freq, self.position.rotary_dim, ctx.new_len,
-                                            table, site.k, site.v, rows_cap, self.query_scale, self.softcap,
-                                            self.window, ctx.dtype, max_keys=ctx.max_keys(site), write_kv=owns_cache)
+                                            table, k_pool, v_pool, rows_cap, self.query_scale, self.softcap,
+                                            self.window, ctx.dtype, max_keys=ctx.max_rows_visible(site), write_kv=owns_cache)
             return ops.linear(out, self.w_o, ctx.dtype, defer=True)
         if owns_cache:
             qkv = ops.linear(x, self.w_qkv, ctx.dtype)
@@ -80,10 +82,10 @@ class Attention(Mixer):
             q, k, v = ops.linear(x, self.w_qkv[:Q], ctx.dtype), None, None
         if ctx.mode == "decode":
             ops.rope_kv_write(q, k, v, H, KV, hd, self.inv_freq, self.position.rotary_dim,
-                              ctx.row_seq, ctx.row_pos, ctx.new_len, table, site.k, site.v, rows_cap, pairing=pairing)
-            out = ops.attention_decode(q, H, KV, hd, ctx.new_len, table, site.k, site.v, rows_cap,
+                              ctx.row_seq, ctx.row_pos, ctx.new_len, table, k_pool, v_pool, rows_cap, pairing=pairing)
+            out = ops.attention_decode(q, H, KV, hd, ctx.new_len, table, k_pool, v_pool, rows_cap,
                                        self.query_scale, self.softcap, self.window, ctx.dtype,
-                                       max_keys=ctx.max_keys(site))
+                                       max_keys=ctx.max_rows_visible(site))
             return ops.linear(out, self.w_o, ctx.dtype, defer=True)
         # Sequences that go on by several tokens (or some start while others go on) see cached positions and the
         # step's own rows.  The attention reads the cached ones where they lie, as earlier steps left them, and the
@@ -91,18 +93,19 @@ class Attention(Mixer):
         # they take the places of positions that the step's earlier queries still see.
         extend = ctx.mode == "extend"
         ops.rope_kv_write(q, k, v, H, KV, hd, self.inv_freq, self.position.rotary_dim,
-                          ctx.row_seq, ctx.row_pos, ctx.new_len, table, site.k, site.v, rows_cap, pairing=pairing,
+                          ctx.row_seq, ctx.row_pos, ctx.new_len, table, k_pool, v_pool, rows_cap, pairing=pairing,
                           write=not extend)
         if owns_cache:
-            ctx.offer_step_kv(k, v)
+            ctx.offer_step_rows(k=k, v=v)
         else:
-            k, v = ctx.step_kv_of(ctx.cache_owner)
+            theirs = ctx.step_rows_of(ctx.cache_owner)
+            k, v = theirs["k"], theirs["v"]
         out = ops.attention_prefill(q, k, v, H, KV, hd, ctx.cu_rows, ctx.max_count,
                                     self.query_scale, self.softcap, self.window, ctx.dtype,
                                     row_seq=ctx.row_seq, row_pos=ctx.row_pos,
-                                    cached=(ctx.new_len, table, site.k, site.v, rows_cap) if extend else None)
+                                    cached=(ctx.new_len, table, k_pool, v_pool, rows_cap) if extend else None)
         if extend and owns_cache:
-            row_seq, row_pos, new_len, k_pool, v_pool = ctx.row_seq, ctx.row_pos, ctx.new_len, site.k, site.v
+            row_seq, row_pos, new_len = ctx.row_seq, ctx.row_pos, ctx.new_len
             ctx.after_readers(lambda: ops.kv_write(k, v, KV, hd, row_seq, row_pos, new_len, table, k_pool, v_pool, rows_cap))
         return ops.linear(out, self.w_o, ctx.dtype, defer=True)
 

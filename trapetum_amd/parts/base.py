@@ -8,7 +8,7 @@ step (`forward`).  Interfaces:
                norm multiplies by, so that blocks can fuse a norm into a neighbour.
   Position     `rotary_dim` and `inv_freq(device)`: the rotation table a mixer applies
                to queries and keys before the cache write.
-  Mixer        cache_spec() -> KVSpec | StateSpec | None;
+  Mixer        cache_spec() -> TokenSpec | StateSpec | None;
                forward(ctx, x, site) -> rows [M, hidden], x being the normed rows.
   FeedForward  forward(ctx, x) -> rows [M, hidden].
                (A mixer or feed-forward may return what `ops.linear(..., defer=True)` gave it: the block
