@@ -115,6 +115,14 @@ def test_bench_line(tmp_path):
     assert set(d["prefill"]) >= {"value", "tokens", "ms", "frac"} and d["prefill"]["tokens"] == 2048
     r = d["roofline"]
     assert r["bound"] == "hbm" and r["unit"] == "GB/s" and r["peak"] == 8000.0 and abs(r["frac"] - r["achieved"] / r["peak"]) < 1e-3
-    assert set(d["points"]) >= {"decode_b1", "decode_b64"}
+    assert set(d["points"]) >= {"decode_b1", "decode_b64", "generate_b8", "decode_b8_ctx7900", "decode_b8_9b", "decode_b8_27b",
+                                "prefill_2048_9b", "prefill_2048_27b"}
+    assert all(isinstance(v, float) and v > 0 for v in d["points"].values())
+    assert set(d["points_frac"]) == set(d["points"]) - {"generate_b8"} and all(0 < v < 1 for v in d["points_frac"].values())
+    k = d["kernels"]
+    assert {"decode_b8.gate_up", "decode_b8.down", "decode_b8.qkv", "decode_b8.o", "decode_b8.add_rms_norm", "prefill_2048.gate_up",
+            "prefill_2048.attention"} <= set(k) and any(n.startswith("decode_b8.attention_ctx") for n in k)
+    for name, row in k.items():
+        assert row["us"] > 0 and 0 < row["frac"] < 1 and ("GB/s" in row) != ("TFLOP/s" in row), name
     p = subprocess.run([sys.executable, "bench.py", "--gpus", "2"], cwd=ROOT, capture_output=True, text=True, timeout=120)
     assert p.returncode == 2 and len((p.stdout + p.stderr).strip().splitlines()) == 1
