@@ -135,6 +135,11 @@ LINEAR_SHAPES += [(1, 77, 8), (2, 301, 1000), (2, 130, 1536), (1, 257, 3584), (2
 LINEAR_SHAPES += [(3, 77, 8), (8, 1001, 2304), (7, 130, 2312), (6, 250, 5000), (4, 4099, 600), (5, 9, 9216)]
 
 
+# nine to 64 rows: every number of 16-row groups of X, an N and a K that end inside a tile and inside a k step, K slices
+# whose number a whole number of k steps makes smaller than was asked for
+LINEAR_SHAPES += [(9, 77, 64), (33, 1001, 2304), (48, 130, 2312), (64, 250, 5000), (20, 4099, 600), (50, 9, 9216), (16, 64, 72)]
+
+
 @pytest.mark.parametrize("algo", [1, 2, 3, 4, 5, 6, 7, 8, 9])
 @pytest.mark.parametrize("m,n,k", LINEAR_SHAPES)
 def test_linear_bf16(ops, algo, m, n, k):
@@ -152,12 +157,14 @@ def test_linear_bf16(ops, algo, m, n, k):
         got_b = ops.linear(x, w, torch.bfloat16)
         got_f = ops.linear(x, w, torch.float32)
         got_c = ops.linear(x, w, torch.float32, softcap=3.0)
+        got_d = ops.rows(ops.linear(x, w, torch.bfloat16, defer=True), torch.float32)      # K slices, where the kernel makes them
     finally:
         ops.force_linear = 0
     ref = x.cpu().double() @ w.cpu().double().T
     assert rel_l2(got_f, ref) < 1e-5
     assert rel_l2(got_b, ref) < 4e-3
     assert rel_l2(got_c, 3.0 * torch.tanh(ref / 3.0)) < 1e-5
+    assert rel_l2(got_d, ref) < 4e-3
 
 
 @pytest.mark.parametrize("dt", ["f32", "bf16"])
@@ -191,7 +198,8 @@ def test_linear_f32(ops, m, n, k):
 @pytest.mark.parametrize("dt", ["bf16", "f32"])
 @pytest.mark.parametrize("m,inter,k", [(1, 16, 16), (4, 200, 88), (40, 320, 96), (9, 1000, 2304), (150, 72, 136),
                                        (150, 72, 128), (700, 1000, 320), (130, 36010, 64), (2, 1000, 2304), (1, 75, 4608),
-                                       (8, 9216, 2304), (3, 41, 2504), (7, 8, 520)])
+                                       (8, 9216, 2304), (3, 41, 2504), (7, 8, 520), (64, 9216, 2304), (33, 1000, 200),
+                                       (17, 41, 2504), (48, 8, 520)])
 def test_gated_linear(ops, algo, dt, m, inter, k):
     if dt == "f32" and algo != 1:
         pytest.skip("float32 runs on the plain kernel only")

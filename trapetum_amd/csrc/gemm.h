@@ -4,6 +4,8 @@
 #include "common.h"
 
 enum { TP_EPI_NONE = 0, TP_EPI_SOFTCAP = 1, TP_EPI_GATED = 2 };
+// steps of 64 k a wave of the 8-row kernel has in flight at once: four waves a block read a K of 2,304 in one round of loads
+#define TP_R8_MAX_STEPS 9
 
 struct GemmArgs {
     const void* x; const void* w; void* y;

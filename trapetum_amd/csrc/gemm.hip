@@ -131,26 +131,37 @@ static int pick(const GemmArgs& a, int algo) {
     // at 8 rows; at 3 and 4 rows, where the choice below is the skinny kernel, 2B logits 250 / 228, 9B gate/up 49.3 / 41.8,
     // 27B gate/up 142 / 127, 27B qkv 16.9 / 19.4.  A slice of K beyond 2,304 takes the kernel a second round of loads.
     // A decode step of 8 sequences at the 2B sizes: 2.30 -> 2.00 ms.
+    // The bounds below are what those measurements have in common, in the kernels' own terms:
+    //   ONE_ROUND_K  the K a block of the 8-row kernel reads in one round of loads (TP_R8_MAX_STEPS steps of 64 k by four
+    //                waves): beyond it the kernel loops, and a slice of K left to the consumer keeps it within one round;
+    //   WIDE_N       from here on a product is the logits' kind: so many rows of W that the tiled kernel's 64 x 64 tiles
+    //                fill every CU several times over (512 tiles = two a CU) and its larger k steps win;
+    //   LARGE_NK     elements of W from which the tiled kernel's streaming wins at 8 rows and more (the 27B matrices and
+    //                every gated product: 340 MB, 93 -> 74 us), measured between 21 M (2B down: the 8-row kernel wins)
+    //                and 42 M (2B gate/up: the tiled kernel wins);
+    //   R8_SLICED_NK elements of W up to which the 8-row kernel, its K in slices for the consumer, beat the tiled kernel
+    //                in a whole step (all the 2B and 9B products but the 9B feed-forward; the 27B ones lose).
+    constexpr int ONE_ROUND_K = TP_R8_MAX_STEPS * 256, WIDE_N = 64 * 512;
+    constexpr long LARGE_NK = 24000000, R8_SLICED_NK = 32000000;
     if (a.M <= 8 && gemm_rows8_supports(a)) {
         const long nk = (long)a.N * a.K;
         if (a.defer && a.epilogue == TP_EPI_NONE) {
-            if (nk <= 32000000) return 5;     // (2B o alone is no faster, 5.0 / 5.2, but a step of 8 sequences is: 2.001 -> 1.988 ms)
+            if (nk <= R8_SLICED_NK) return 5;     // (2B o alone is no faster, 5.0 / 5.2, but a step of 8 sequences is: 2.001 -> 1.988 ms)
         } else if (a.M < 8) {
-            if (a.epilogue == TP_EPI_GATED || a.K <= 2304 || a.N >= 32768) return 5;
-        } else if (a.K <= 2304 && a.N < 32768) {
+            if (a.epilogue == TP_EPI_GATED || a.K <= ONE_ROUND_K || a.N >= WIDE_N) return 5;
+        } else if (a.K <= ONE_ROUND_K && a.N < WIDE_N) {
             return 5;
         }
     }
     if (gemm_mfma_supports(a)) {
         const bool sliced = a.defer && a.epilogue == TP_EPI_NONE;
-        // (up to 16 rows the tiled kernel's lead on qkv and down is lost again in their consumers, which then add
-        // 9 and 16 slices instead of 2 and 4: a decode step of 8 sequences took 2.40 ms instead of 2.26; a single
-        // sequence is faster on the skinny kernel throughout)
-        // (from 8 rows on the large matrices gain more than that: 27B down, 340 MB, 93 -> 74 us; a 27B step of 8
-        // sequences 14.2 -> 13.65 ms)
-        if (a.M >= 8 && (a.epilogue == TP_EPI_GATED || (long)a.N * a.K >= 24000000)) return 3;
-        if (a.M >= 8 && a.N >= 32768) return 3;
-        if (a.M > 16 && (sliced || a.N >= 8192)) return 3;
+        // (at 8 rows the tiled kernel's lead on qkv and down is lost again in their consumers, which then add 9 and 16
+        // slices instead of 2 and 4; a single sequence is faster on the skinny kernel throughout)
+        if (a.M >= 8 && (a.epilogue == TP_EPI_GATED || (long)a.N * a.K >= LARGE_NK)) return 3;
+        if (a.M >= 8 && a.N >= WIDE_N) return 3;
+        // from 9 rows on the tiled kernel wins every product of a layer against the skinny one (2B, 16 rows, cold
+        // weights: qkv 6.4 / 8.0 us, o 5.1 / 5.3, down 11.5 / 18.6; a step of 16 sequences 2.47 -> 2.32 ms)
+        if (a.M > 8 && (sliced || a.N >= 8192)) return 3;
     }
     if (gemm_skinny_supports(a)) return 2;
     if (gemm_mfma_supports(a)) return 3;

@@ -381,8 +381,20 @@ static Plan plan_of(const GemmArgs& a) {
     return mid_tile_plan(a, may_slice);
 }
 
+// The plan with its slices as the launch makes them: a slice is a whole number of k steps, so fewer slices than were asked
+// for may cover K (K 9216 in 16 slices: steps of 128 make 15 of 640), and the consumer must add exactly those written.
+static Plan final_plan(const GemmArgs& a) {
+    Plan p = plan_of(a);
+    if (p.splits > 1) {
+        const int kstep = p.tile.tm == 2 ? SMALL_KS : BK;
+        const int kps = tp_cdiv(tp_cdiv(a.K, p.splits), kstep) * kstep;
+        p.splits = tp_cdiv(a.K, kps);
+    }
+    return p;
+}
+
 // K slices for products whose tiles alone do not fill the chip and whose consumer adds the slices (defer)
-int gemm_mfma_splits(const GemmArgs& a) { return plan_of(a).splits; }
+int gemm_mfma_splits(const GemmArgs& a) { return final_plan(a).splits; }
 
 template <int EPI, int TM, int TN, int KS = BK>
 static void mfma_launch(const GemmArgs& a, void* y, int out_dtype, int splits, int kps) {
@@ -426,7 +438,7 @@ int gemm_mfma_launch(const GemmArgs& a) {
     TP_REQUIRE(((uintptr_t)a.x % 16 == 0) && ((uintptr_t)a.w % 16 == 0), "tiled product: operands must be 16-byte aligned");
     TP_REQUIRE(a.K < (1 << 22), "tiled product: K=%d exceeds the kernel's 32-bit offsets", a.K);
     TP_REQUIRE((long)tp_cdiv(a.M, 64) * tp_cdiv(a.N, 64) < (1L << 31), "tiled product: too many tiles for one launch (M=%d N=%d)", a.M, a.N);
-    const Plan plan = plan_of(a);
+    const Plan plan = final_plan(a);
     const Tile t = plan.tile;
     const int splits = plan.splits;
     if (splits > 1) {

@@ -19,7 +19,7 @@ typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
 
 namespace {
-constexpr int R8_MAX_STEPS = 9;                  // steps of 64 k a wave has in flight at once: a K slice of 2,304 in one go
+constexpr int R8_MAX_STEPS = TP_R8_MAX_STEPS;    // steps of 64 k a wave has in flight at once: a K slice of 2,304 in one go
 union Frag8 { uint4 u; bf16x8 v; };
 }
 
@@ -140,7 +140,7 @@ static int rows8_groups(const GemmArgs& a) {
     const int most = a.defer && a.epilogue == TP_EPI_NONE && a.K / 512 > 1 ? a.K / 512 : 1;
     if (!a.defer) return (long)tp_cdiv(a.N, 16) >= 256 ? 2 : 1;
     for (int g = 4; g > 1; g >>= 1)             // (2B step of 8 sequences with at most 4 / 2 / 1 groups: 2.001 / 2.024 / 2.062 ms)
-        if ((long)tp_cdiv(a.N, 8 * g) * most >= 768) return g;
+        if ((long)tp_cdiv(a.N, 8 * g) * most >= 3 * 256) return g;      // three blocks for each of the chip's 256 CUs
     return 1;
 }
 
