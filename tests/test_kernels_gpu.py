@@ -140,7 +140,7 @@ LINEAR_SHAPES += [(3, 77, 8), (8, 1001, 2304), (7, 130, 2312), (6, 250, 5000), (
 LINEAR_SHAPES += [(9, 77, 64), (33, 1001, 2304), (48, 130, 2312), (64, 250, 5000), (20, 4099, 600), (50, 9, 9216), (16, 64, 72)]
 
 
-@pytest.mark.parametrize("algo", [1, 2, 3, 4, 5, 6, 7, 8, 9])
+@pytest.mark.parametrize("algo", [1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11])
 @pytest.mark.parametrize("m,n,k", LINEAR_SHAPES)
 def test_linear_bf16(ops, algo, m, n, k):
     if algo in (8, 9) and k % 64:
@@ -194,7 +194,7 @@ def test_linear_f32(ops, m, n, k):
     assert torch.equal(alone[0], got[m - 1])
 
 
-@pytest.mark.parametrize("algo", [1, 2, 3, 4, 5, 6, 8])
+@pytest.mark.parametrize("algo", [1, 2, 3, 4, 5, 6, 8, 10, 11])
 @pytest.mark.parametrize("dt", ["bf16", "f32"])
 @pytest.mark.parametrize("m,inter,k", [(1, 16, 16), (4, 200, 88), (40, 320, 96), (9, 1000, 2304), (150, 72, 136),
                                        (150, 72, 128), (700, 1000, 320), (130, 36010, 64), (2, 1000, 2304), (1, 75, 4608),

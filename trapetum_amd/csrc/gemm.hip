@@ -107,14 +107,14 @@ static int check_args(const GemmArgs& a) {
 }
 
 // algo: 0 = choose, 1 = plain, 2 = skinny matrix-core, 3 = tiled matrix-core (6: with its wide tile, 7: with its 128 x 96 tile,
-// 8, 9: with its loop that loads straight into LDS, 128 x 128 and 128 x 96), 4 = multiply-adds for one or two rows,
-// 5 = matrix-core kernel for up to eight rows
+// 8, 9: with its loop that loads straight into LDS, 128 x 128 and 128 x 96; 10, 11: its 64 x 32 and 64 x 64 tiles with two k
+// steps asked for ahead), 4 = multiply-adds for one or two rows, 5 = matrix-core kernel for up to eight rows
 static int pick(const GemmArgs& a, int algo) {
     if (algo == 1) return 1;
     if (algo == 4) return gemv_supports(a) ? 4 : -4;
     if (algo == 5) return gemm_rows8_supports(a) ? 5 : -5;
     if (algo == 2) return gemm_skinny_supports(a) ? 2 : -2;
-    if (algo == 3 || algo == 6 || algo == 7 || algo == 8 || algo == 9) return gemm_mfma_supports(a) ? 3 : -3;
+    if (algo == 3 || (algo >= 6 && algo <= 11)) return gemm_mfma_supports(a) ? 3 : -3;
     // Up to 64 rows both matrix-core kernels stream W once; which is faster was measured on MI355X at the 2B shapes
     // (cold weights, microseconds, skinny / tiled with 64 x 64 tiles and k steps of 128):
     //   logits  N 256000            8 rows 277 / 222

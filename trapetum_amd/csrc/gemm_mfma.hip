@@ -1,7 +1,7 @@
 // bf16 product for many rows (prefill) and for few rows of a wide or large matrix: LDS-tiled, on the matrix cores,
 // fp32 accumulation.
 //
-// Block: 256 threads = 4 waves in a 2 x 2 arrangement over a tile of Y (128 x 128, 128 x 96, 128 x 256 or 64 x 64); each
+// Block: 256 threads = 4 waves in a 2 x 2 arrangement over a tile of Y (128 x 128, 128 x 96, 128 x 256 or 64 x 64; 4 x 1 over 64 x 32); each
 // wave owns TM x TN tiles of v_mfma_f32_16x16x32_bf16.  W rows are the A operand and X rows the B operand (both are
 // contiguous along k, which is what the instruction wants per lane), so a lane ends up with 4 consecutive columns of
 // one row of Y (one 8- or 16-byte store), and with the gate and the up column of the same unit in two accumulators of
@@ -80,20 +80,24 @@ __device__ __forceinline__ void store_tile(const f32x4 (&acc)[TM][TN], void* __r
 }
 
 // TM x TN: the 16 x 16 tiles of a wave; the block's 2 x 2 waves cover BM = 32 TM rows of X and BN = 32 TN rows of W
+// WM: waves along the rows of X (2: the 2 x 2 arrangement; 4: four waves over 64 rows of X, one wave across the tile's rows of W)
+// DEEP: two k steps are asked for ahead, in two sets of staging registers (tiles that stream W for few rows)
 // SHORT: whole tiles load their k steps by the short path described below
 // KS: elements of a k step (64, or 128 for the 64 x 64 tiles, which stream W and are bound by the bytes a block has
 // in flight: one step ahead is all a block asks for)
-template <int EPI, int TM, int TN, bool SHORT, int KS = BK>
+template <int EPI, int TM, int TN, bool SHORT, int KS = BK, int WM = 2, bool DEEP = false>
 __global__ void __launch_bounds__(256, 2)
 gemm_mfma_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __restrict__ Y,
             int M, int N, int K, int m_tiles, int out_dtype, float2 epi, int units, int k_per_split, int xcd_panels) {
-    constexpr int BM = 32 * TM, BN = 32 * TN, BK = KS, LDS = KS, CPR = KS / 8, LA = TM * KS / 64, LB = TN * KS / 64;
+    constexpr int WN = 4 / WM, BM = 16 * WM * TM, BN = 16 * WN * TN, BK = KS, LDS = KS, CPR = KS / 8;
+    constexpr int LA = BM * KS / 2048, LB = BN * KS / 2048;    // 16-byte chunks of a step's tile per thread
+    static_assert(BM * KS % 2048 == 0 && BN * KS % 2048 == 0, "a step's tile is a whole number of chunks per thread");
     constexpr int SWZ = CPR >= 16 ? 15 : 7;        // rows 256 bytes long all start at one bank: their 16 chunks are permuted as a whole
-    static_assert(!SHORT || KS == 64, "the short load path is written for steps of 64");
+    static_assert(!SHORT || (KS == 64 && WM == 2), "the short load path is written for steps of 64 and 2 x 2 waves");
     __shared__ __attribute__((aligned(16))) bf16_t As[BM * LDS];
     __shared__ __attribute__((aligned(16))) bf16_t Bs[BN * LDS];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 15, g = lane >> 4;
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = WM == 4 ? wave : wave >> 1, wn = WM == 4 ? 0 : wave & 1;
     // Block ids go to the chip's 8 XCDs in turn, and each XCD has an L2 of its own.  On a large grid an XCD therefore
     // takes a contiguous range of the tiles, walked in panels of four N tiles (M tiles of a panel one after another, its
     // N tiles fastest), so that the blocks an XCD runs together share their W and X tiles in its L2.  Measured on the
@@ -124,30 +128,31 @@ gemm_mfma_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __
     // row per chunk; only a last, partial step tests every chunk.  A launch without a whole tile (fewer rows than a tile has) and the 64 x 64 tiles,
     // which stream W, run without the short path compiled in: its mere presence costs them a fifth (27B gate/up at 64
     // rows in 128 x 128 tiles: 188 against 149 us), while whole large tiles gain a twentieth from it.
-    bf16x8 ra[LA], rb[LB];
+    constexpr int SETS = DEEP ? 2 : 1;             // register sets of staged chunks: k steps asked for ahead
+    bf16x8 ra[SETS][LA], rb[SETS][LB];
     const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
     const bool inner = SHORT && m0 + BM <= M && n0 + BN <= N;
     const unsigned xoff = (unsigned)(tid >> 3) * (unsigned)K * 2u + (unsigned)(tid & 7) * 16u;      // the same for X and W
     const size_t rows32 = (size_t)32 * K * 2;
     const char* const x_origin = reinterpret_cast<const char*>(X + (size_t)m0 * K);
     const char* const w_origin = reinterpret_cast<const char*>(W + (size_t)n0 * K);
-    auto fetch = [&](int k0) {
+    auto fetch = [&](bf16x8 (&ra)[LA], bf16x8 (&rb)[LB], int k0) {
         if (inner && k0 + BK <= k_end) {
             const char* const xb = x_origin + (size_t)k0 * 2, * const wb = w_origin + (size_t)k0 * 2;
             const unsigned off = in_register(xoff);
 #pragma unroll
-            for (int i = 0; i < TM; i++) ra[i] = *reinterpret_cast<const bf16x8*>(xb + i * rows32 + off);
+            for (int i = 0; i < LA; i++) ra[i] = *reinterpret_cast<const bf16x8*>(xb + i * rows32 + off);
 #pragma unroll
-            for (int i = 0; i < TN; i++) rb[i] = *reinterpret_cast<const bf16x8*>(wb + i * rows32 + off);
+            for (int i = 0; i < LB; i++) rb[i] = *reinterpret_cast<const bf16x8*>(wb + i * rows32 + off);
         } else if (SHORT && k0 + BK <= k_end) {
             // a tile over the edge of Y: a row past the edge reads the tile's last row (its products are never stored)
             const char* const xb = x_origin + (size_t)k0 * 2, * const wb = w_origin + (size_t)k0 * 2;
             const unsigned chunk = in_register((unsigned)(tid & 7) * 16u), row_bytes = (unsigned)K * 2u;
 #pragma unroll
-            for (int i = 0; i < TM; i++)
+            for (int i = 0; i < LA; i++)
                 ra[i] = *reinterpret_cast<const bf16x8*>(xb + ((unsigned)min((tid >> 3) + 32 * i, M - 1 - m0) * row_bytes + chunk));
 #pragma unroll
-            for (int i = 0; i < TN; i++)
+            for (int i = 0; i < LB; i++)
                 rb[i] = *reinterpret_cast<const bf16x8*>(wb + ((unsigned)min((tid >> 3) + 32 * i, N - 1 - n0) * row_bytes + chunk));
         } else {
 #pragma unroll
@@ -162,7 +167,7 @@ gemm_mfma_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __
             }
         }
     };
-    auto stage = [&]() {
+    auto stage = [&](const bf16x8 (&ra)[LA], const bf16x8 (&rb)[LB]) {
 #pragma unroll
         for (int i = 0; i < LA; i++) {
             const int c = tid + i * 256, row = c / CPR, kc = ((c % CPR) ^ (row & SWZ)) * 8;  // chunk j of a row sits at j ^ (row & SWZ)
@@ -180,13 +185,7 @@ gemm_mfma_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __
     for (int i = 0; i < TM; i++)
 #pragma unroll
         for (int j = 0; j < TN; j++) acc[i][j] = (f32x4){0.f, 0.f, 0.f, 0.f};
-
-    fetch(k_begin);
-    for (int k0 = k_begin; k0 < k_end; k0 += BK) {
-        __syncthreads();                       // everyone is done reading the previous tile
-        stage();
-        __syncthreads();
-        if (k0 + BK < k_end) fetch(k0 + BK);
+    auto products = [&]() {
 #pragma unroll
         for (int ks = 0; ks < BK; ks += 32) {
             Frag a[TM], b[TN];
@@ -201,6 +200,21 @@ gemm_mfma_k(const bf16_t* __restrict__ X, const bf16_t* __restrict__ W, void* __
                 for (int j = 0; j < TN; j++)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b[j].v, a[i].v, acc[i][j], 0, 0, 0);
         }
+    };
+    // one step: the set's chunks to LDS, the set refilled `SETS` steps ahead, the step's products
+    auto step = [&](bf16x8 (&ra)[LA], bf16x8 (&rb)[LB], int k0) {
+        __syncthreads();                       // everyone is done reading the previous tile
+        stage(ra, rb);
+        __syncthreads();
+        if (k0 + SETS * BK < k_end) fetch(ra, rb, k0 + SETS * BK);
+        products();
+    };
+
+    fetch(ra[0], rb[0], k_begin);
+    if (DEEP && k_begin + BK < k_end) fetch(ra[SETS - 1], rb[SETS - 1], k_begin + BK);
+    for (int k0 = k_begin; k0 < k_end; k0 += SETS * BK) {
+        step(ra[0], rb[0], k0);
+        if (DEEP && k0 + BK < k_end) step(ra[SETS - 1], rb[SETS - 1], k0 + BK);
     }
 
     store_tile<EPI, TM, TN>(acc, Y, M, N, m0, n0, wm, wn, r, g, out_dtype, epi, units);
@@ -311,7 +325,7 @@ bool gemm_mfma_supports(const GemmArgs& a) {
 // straight into LDS where K allows it; the register-staged loop also has 128 x 256 tiles (less LDS traffic per matrix
 // instruction; two blocks fit a CU) for grids of at least four rounds of those 512 places (2B gate/up, register-staged:
 // 930 against 790 TFLOP/s at 8192 rows, 700 against 790 at 2048).
-struct Tile { int tm, tn; };
+struct Tile { int tm, tn, wm = 2; bool deep = false; };        // wm: waves along the rows of X (2 x 2 or 4 x 1)
 struct Plan { Tile tile; int splits; bool direct = false; };
 
 // K slices of a product of few rows, which is bound by reading W and wants every CU streaming.  From 17 rows on one
@@ -366,7 +380,9 @@ static Plan mid_tile_plan(const GemmArgs& a, bool may_slice) {
 }
 
 static Plan plan_of(const GemmArgs& a) {
-    const bool may_slice = a.defer && a.epilogue == TP_EPI_NONE && a.algo < 6;
+    const bool may_slice = a.defer && a.epilogue == TP_EPI_NONE && (a.algo < 6 || a.algo == 11);
+    if (a.algo == 10) return {{1, 2, 4, true}, 1};
+    if (a.algo == 11) return {{2, 2, 2, true}, may_slice ? small_tile_splits(a, (long)tp_cdiv(a.M, 64) * tp_cdiv(a.N, 64)) : 1};
     if (a.algo == 6) return {{4, 8}, 1};
     if (a.algo == 7) return {{4, a.epilogue == TP_EPI_GATED ? 4 : 3}, 1};
     if (a.algo == 8) return {{4, 4}, 1, true};
@@ -374,8 +390,19 @@ static Plan plan_of(const GemmArgs& a) {
     // the logits of 64 rows: 250 us with 128 x 128, 275 with 64 x 64; up to 256 rows of a narrow product: 128 x 128
     // tiles would leave most CUs idle (down at 128 rows: 44 us on 72 blocks, against 15 us at 64 rows on 576 blocks
     // of 64 x 64; at 512 rows 128 x 128 wins again)
-    if ((a.M <= 64 && !(a.M > 32 && a.N >= 32768)) || (a.M <= 256 && (long)tp_cdiv(a.M, 128) * tp_cdiv(a.N, 128) < 256))
-        return {{2, 2}, may_slice ? small_tile_splits(a, (long)tp_cdiv(a.M, 64) * tp_cdiv(a.N, 64)) : 1};
+    if ((a.M <= 64 && !(a.M > 32 && a.N >= 32768)) || (a.M <= 256 && (long)tp_cdiv(a.M, 128) * tp_cdiv(a.N, 128) < 256)) {
+        const long tiles = (long)tp_cdiv(a.M, 64) * tp_cdiv(a.N, 64);
+        Tile t{2, 2};
+        // Up to 32 rows what such a product waits for is W, and a block that asks one k step ahead has 16 KB of it in
+        // flight: with two steps ahead (a second set of staging registers) the long loops gain, those of a gated product
+        // (never sliced) and of the slices of 17 rows and more (2B gate/up at 16 rows 27.6 -> 23.0 us, 27B at 8 rows
+        // 141 -> 126, 9B qkv at 32 rows 21.1 -> 18.1); slices of a few steps (up to 16 rows) and 64 rows do not.
+        // A gated product with about a block a CU in these tiles gains more from 64 x 32 tiles, twice the blocks with
+        // the same bytes in flight each (2B gate/up at 8 to 24 rows: 27.7 -> 22.5 us; the 9B and 27B shapes do not).
+        if (a.M <= 32 && (a.epilogue == TP_EPI_GATED || (may_slice && a.M > 16))) t.deep = true;
+        if (a.M <= 32 && a.epilogue == TP_EPI_GATED && tiles <= 320) t = {1, 2, 4, true};
+        return {t, may_slice ? small_tile_splits(a, tiles) : 1};
+    }
     // register-staged loop only: 128 x 256 tiles from four rounds of their 512 places on
     if (!direct_ok(a) && (long)tp_cdiv(a.M, 128) * tp_cdiv(a.N, 256) >= 2048) return {{4, 8}, 1};
     return mid_tile_plan(a, may_slice);
@@ -386,7 +413,7 @@ static Plan plan_of(const GemmArgs& a) {
 static Plan final_plan(const GemmArgs& a) {
     Plan p = plan_of(a);
     if (p.splits > 1) {
-        const int kstep = p.tile.tm == 2 ? SMALL_KS : BK;
+        const int kstep = p.tile.tm <= 2 ? SMALL_KS : BK;
         const int kps = tp_cdiv(tp_cdiv(a.K, p.splits), kstep) * kstep;
         p.splits = tp_cdiv(a.K, kps);
     }
@@ -396,17 +423,17 @@ static Plan final_plan(const GemmArgs& a) {
 // K slices for products whose tiles alone do not fill the chip and whose consumer adds the slices (defer)
 int gemm_mfma_splits(const GemmArgs& a) { return final_plan(a).splits; }
 
-template <int EPI, int TM, int TN, int KS = BK>
+template <int EPI, int TM, int TN, int KS = BK, int WM = 2, bool DEEP = false>
 static void mfma_launch(const GemmArgs& a, void* y, int out_dtype, int splits, int kps) {
-    const int m_tiles = tp_cdiv(a.M, 32 * TM), n_tiles = tp_cdiv(a.N, 32 * TN);
+    const int m_tiles = tp_cdiv(a.M, 16 * WM * TM), n_tiles = tp_cdiv(a.N, 16 * (4 / WM) * TN);
     dim3 grid((unsigned)(m_tiles * n_tiles), splits);
     const int xcd_panels = (long)m_tiles * n_tiles >= 1024 ? 1 : 0;
     if (TM > 2 && a.M >= 32 * TM && a.N >= 32 * TN)
         gemm_mfma_k<EPI, TM, TN, (TM > 2), KS><<<grid, 256, 0, a.stream>>>((const bf16_t*)a.x, (const bf16_t*)a.w, y, a.M, a.N, a.K, m_tiles,
                                                                       out_dtype, epi_constants(a), a.units, kps, xcd_panels);
     else
-        gemm_mfma_k<EPI, TM, TN, false, KS><<<grid, 256, 0, a.stream>>>((const bf16_t*)a.x, (const bf16_t*)a.w, y, a.M, a.N, a.K, m_tiles,
-                                                                   out_dtype, epi_constants(a), a.units, kps, xcd_panels);
+        gemm_mfma_k<EPI, TM, TN, false, KS, WM, DEEP><<<grid, 256, 0, a.stream>>>((const bf16_t*)a.x, (const bf16_t*)a.w, y, a.M, a.N, a.K, m_tiles,
+                                                                       out_dtype, epi_constants(a), a.units, kps, xcd_panels);
 }
 
 template <int EPI>
@@ -426,7 +453,9 @@ static void mfma_launch_direct(const GemmArgs& a, Tile t, void* y, int out_dtype
 
 template <int EPI>
 static void mfma_launch_tile(const GemmArgs& a, Tile t, void* y, int out_dtype, int splits, int kps) {
-    if (t.tm == 2) mfma_launch<EPI, 2, 2, SMALL_KS>(a, y, out_dtype, splits, kps);
+    if (t.wm == 4) mfma_launch<EPI, 1, 2, SMALL_KS, 4, true>(a, y, out_dtype, splits, kps);
+    else if (t.tm == 2 && t.deep) mfma_launch<EPI, 2, 2, SMALL_KS, 2, true>(a, y, out_dtype, splits, kps);
+    else if (t.tm == 2) mfma_launch<EPI, 2, 2, SMALL_KS>(a, y, out_dtype, splits, kps);
     else if (t.tn == 8) mfma_launch<EPI, 4, 8>(a, y, out_dtype, splits, kps);
     else if (t.tn == 3) {
         if constexpr (EPI != TP_EPI_GATED) mfma_launch<EPI, 4, 3>(a, y, out_dtype, splits, kps);
@@ -444,7 +473,7 @@ int gemm_mfma_launch(const GemmArgs& a) {
     if (splits > 1) {
         const size_t need = (size_t)splits * a.M * a.N * sizeof(float);
         TP_REQUIRE(a.workspace && a.workspace_bytes >= need, "tiled product: workspace of %zu bytes, %zu needed", a.workspace_bytes, need);
-        const int kstep = t.tm == 2 ? SMALL_KS : BK;
+        const int kstep = t.tm <= 2 ? SMALL_KS : BK;
         const int kps = tp_cdiv(tp_cdiv(a.K, splits), kstep) * kstep;
         if (plan.direct) mfma_launch_direct<TP_EPI_NONE>(a, t, a.workspace, TP_F32, tp_cdiv(a.K, kps), kps);
         else mfma_launch_tile<TP_EPI_NONE>(a, t, a.workspace, TP_F32, tp_cdiv(a.K, kps), kps);

@@ -96,7 +96,7 @@ class HipOps:
         self._sample_ws = {}
         from .. import flags
         plain = flags.force_plain()
-        self.force_linear = 1 if plain else 0   # 1 plain, 2 skinny, 3 tiled (6: its wide tile, 7: its 128 x 96 tile, 8, 9: loads into LDS, 128 x 128 and 128 x 96), 4 multiply-adds (1-2 rows)
+        self.force_linear = 1 if plain else 0   # 1 plain, 2 skinny, 3 tiled (6: its wide tile, 7: its 128 x 96 tile, 8, 9: loads into LDS, 128 x 128 and 128 x 96; 10, 11: 64 x 32 and 64 x 64 tiles, two k steps ahead), 4 multiply-adds (1-2 rows), 5 blocks of 8 rows of W
         self.force_plain_attention = plain
         self._timed = None                      # with TRAPETUM_AMD_PROFILE=1: [(entry point, start event, end event)] not yet summed
         self._profile_totals = {}               # entry point -> (milliseconds, calls)
