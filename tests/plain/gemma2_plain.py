@@ -61,17 +61,22 @@ def rope_inv_freq(head_dim, theta, dtype):
     return 1.0 / (theta ** (torch.arange(0, head_dim, 2, dtype=dtype) / head_dim))
 
 
-def rope(x, positions, theta):
+def rope(x, positions, theta, angle_dtype=None):
     """Rotate-half RoPE on x [T, heads, head_dim] at integer `positions` [T].
 
     Pair (d, d + head_dim/2), angle = pos * inv_freq[d]:
     x[d]' = x[d] cos - x[d+half] sin ; x[d+half]' = x[d+half] cos + x[d] sin.
     runtime/cuda/codebook_gemv.cu:219-230.
+    `angle_dtype`: the width the table and the angle are formed in.  The reference forms both in 32-bit
+    (model/export_gemma.py:53 `.float()`, codebook_gemv.cu:225 `(float)pos * inv_freq[d]`), whose rounding of an
+    angle of some thousand radians is about pos * 1e-7: nothing at the positions of a short test, a few 1e-5 of the
+    logits at positions beyond 4,000.  None: exact angles in x's own width.
     """
     hd = x.shape[-1]
     half = hd // 2
-    inv = rope_inv_freq(hd, theta, x.dtype)
-    ang = positions.to(x.dtype)[:, None] * inv[None, :]          # [T, half]
+    adt = angle_dtype or x.dtype
+    inv = rope_inv_freq(hd, theta, adt)
+    ang = (positions.to(adt)[:, None] * inv[None, :]).to(x.dtype)      # [T, half]
     c, s = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
     x0, x1 = x[..., :half], x[..., half:]
     return torch.cat([x0 * c - x1 * s, x1 * c + x0 * s], dim=-1)
@@ -127,7 +132,7 @@ def embed(tokens, table, hidden):
     return table[tokens] * math.sqrt(hidden)
 
 
-def attention_block(x, positions, W, p, cfg, window, rnd):
+def attention_block(x, positions, W, p, cfg, window, rnd, angle_dtype=None):
     """q/k/v projections, RoPE on q and k, attention, output projection.  runtime/src/lib.rs:4483-4496."""
     T = x.shape[0]
     H, KV, hd = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
@@ -135,7 +140,7 @@ def attention_block(x, positions, W, p, cfg, window, rnd):
     k = rnd(x @ W[p + "self_attn.k_proj.weight"].T).reshape(T, KV, hd)
     v = rnd(x @ W[p + "self_attn.v_proj.weight"].T).reshape(T, KV, hd)
     theta = float(cfg.get("rope_theta", 10000.0))
-    q, k = rnd(rope(q, positions, theta)), rnd(rope(k, positions, theta))
+    q, k = rnd(rope(q, positions, theta, angle_dtype)), rnd(rope(k, positions, theta, angle_dtype))
     scale = 1.0 / math.sqrt(cfg["query_pre_attn_scalar"])
     a = rnd(attention(q, k, v, scale, cfg.get("attn_logit_softcapping"), window))
     return a.reshape(T, H * hd) @ W[p + "self_attn.o_proj.weight"].T
@@ -150,7 +155,7 @@ def layer_window(cfg, layer):
     return cfg["sliding_window"] if layer % 2 == 0 else None
 
 
-def block(x, positions, W, layer, cfg, rnd):
+def block(x, positions, W, layer, cfg, rnd, angle_dtype=None):
     """x += post_attn_norm(attn(input_norm(x))); x += post_ff_norm(mlp(pre_ff_norm(x))).
 
     runtime/src/lib.rs:4527-4540.
@@ -158,7 +163,7 @@ def block(x, positions, W, layer, cfg, rnd):
     p = f"model.layers.{layer}."
     eps = cfg["rms_norm_eps"]
     n = rnd(rms_norm(x, W[p + "input_layernorm.weight"], eps))
-    a = rnd(attention_block(n, positions, W, p, cfg, layer_window(cfg, layer), rnd))
+    a = rnd(attention_block(n, positions, W, p, cfg, layer_window(cfg, layer), rnd, angle_dtype))
     x = x + rms_norm(a, W[p + "post_attention_layernorm.weight"], eps)
     n = rnd(rms_norm(x, W[p + "pre_feedforward_layernorm.weight"], eps))
     m = rnd(geglu(n, W[p + "mlp.gate_proj.weight"], W[p + "mlp.up_proj.weight"],
@@ -174,14 +179,15 @@ def head(x, W, cfg, rnd):
     return softcap(z, cfg.get("final_logit_softcapping"))
 
 
-def forward(cfg, W, tokens, rnd=None, first_position=0):
-    """Logits [T, vocab] at every position of one whole sequence.  runtime/src/lib.rs:4553-4562."""
+def forward(cfg, W, tokens, rnd=None, first_position=0, angle_dtype=None):
+    """Logits [T, vocab] at every position of one whole sequence.  runtime/src/lib.rs:4553-4562.
+    `angle_dtype`: see rope()."""
     rnd = rnd or (lambda t: t)
     tokens = torch.as_tensor(tokens, dtype=torch.long)
     positions = torch.arange(first_position, first_position + len(tokens))
     x = embed(tokens, W["model.embed_tokens.weight"], cfg["hidden_size"])
     for layer in range(cfg["num_hidden_layers"]):
-        x = block(x, positions, W, layer, cfg, rnd)
+        x = block(x, positions, W, layer, cfg, rnd, angle_dtype)
     return head(x, W, cfg, rnd)
 
 

@@ -180,7 +180,7 @@ def test_post_norms_stand_on_the_sub_layers_outputs(folder_b):
     ref, got = plain.forward(cfg, w, toks), plain.forward(cfg, w8, toks)
     assert rel_l2(got, ref) < 1e-3, rel_l2(got, ref)
 
-    def post_norm_on_the_input(x, positions, W, layer, c, rnd):     # the mistake: it passes the factor on
+    def post_norm_on_the_input(x, positions, W, layer, c, rnd, angle_dtype=None):     # the mistake: it passes the factor on
         p = f"model.layers.{layer}."
         n = plain.rms_norm(plain.rms_norm(x, W[p + "input_layernorm.weight"], c["rms_norm_eps"]), W[p + "post_attention_layernorm.weight"], c["rms_norm_eps"])
         x = x + plain.attention_block(n, positions, W, p, c, plain.layer_window(c, layer), rnd)

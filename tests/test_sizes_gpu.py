@@ -281,10 +281,18 @@ def test_the_real_windows_edge_with_a_key_that_stands_out():
         s = e.cache.acquire()                                # and the whole prompt in one step
         rows.append(e.model.step(e.cache, [s], toks, counts=[len(toks)], want=[P + 4094, P + 4095, P + 4096, P + 4097]))
         out[dt] = torch.cat(rows).float().cpu()
+        if dt == "float32":                                  # what the plain implementation makes of the same tensors
+            from .plain import gemma2_plain as plain
+            # (angles formed in 32-bit, as the reference and the engine form them: at these positions their rounding
+            # alone moves the logits by some 1e-5)
+            truth = plain.forward(cfg.to_dict(), {name: w.double() for name, w in t.items()}, toks, angle_dtype=torch.float32)
         del e, model
         torch.cuda.empty_cache()
     ref, got = out["float32"], out["bfloat16"]
     base = P + 4089                                          # row r of the decoded part is position base + r
+    # the float32 engine at the edge is what the plain implementation (the whole sequence at once, no cache, no ring) gives
+    for r in range(ref.shape[0] - 4):
+        assert rel_l2(ref[r].double(), truth[base + r]) < 1e-5, r
     inside, outside = ref[P + 4095 - base], ref[P + 4096 - base]
     # the planted key matters: the same query token gives other logits once the key has left the window
     assert rel_l2(inside, outside) > 0.2, rel_l2(inside, outside)
