@@ -53,6 +53,31 @@ def test_random_run_generate(tmp_path):
     assert out.strip() == f"continuation ids: {want[1][:want[1].index(want[1][3])]}"
 
 
+def test_a_text_prompt_goes_through_the_folders_tokenizer(tmp_path):
+    """`run DIR --prompt "text"`: the ids are the tokenizer.json's (no special tokens added, as the reference's server
+    encodes: runtime/src/bin/serve.rs:312), the continuation is the one the same ids give, and it comes back as ids and
+    as text; a folder without a tokenizer.json refuses a text prompt with an error that names the file."""
+    from tokenizers import Tokenizer
+    from tokenizers.models import WordLevel
+    from tokenizers.pre_tokenizers import Whitespace
+    config = tmp_path / "config.json"
+    config.write_text(json.dumps(dict(TINY_A, architectures=["Gemma2ForCausalLM"])))
+    folder = tmp_path / "model"
+    cli("random", "--config", config, "--out", folder, "--seed", 3)
+    p = subprocess.run([sys.executable, "-m", "trapetum_amd", "run", str(folder), "--prompt", "w5 w17 w3"], cwd=ROOT,
+                       capture_output=True, text=True, timeout=300)
+    assert p.returncode != 0 and "tokenizer.json" in p.stderr
+    vocab = {f"w{i}": i for i in range(TINY_A["vocab_size"])}
+    tok = Tokenizer(WordLevel(vocab, unk_token="w0"))
+    tok.pre_tokenizer = Whitespace()
+    tok.save(str(folder / "tokenizer.json"))
+    by_ids = cli("run", folder, "--prompt-ids", "5,17,3,9", "--max-tokens", 6, "--dtype", "float32", "--no-stop").strip()
+    by_text = cli("run", folder, "--prompt", "w5 w17 w3 w9", "--max-tokens", 6, "--dtype", "float32", "--no-stop").strip().splitlines()
+    assert by_text[0] == by_ids
+    ids = json.loads(by_ids.split(":", 1)[1])
+    assert by_text[1] == "continuation text: " + " ".join(f"w{i}" for i in ids)
+
+
 def test_float32_weights_are_kept_as_drawn(tmp_path):
     """`random --store-dtype float32` stores the drawn values unrounded, and the float32 engine keeps them so: its
     logits follow a plain run on the unrounded values, not one on their bfloat16 roundings."""

@@ -5,6 +5,7 @@ with the prompt as little-endian int32 ids (runtime/src/bin/gemma_run.rs:1-19, r
 its request options are max_tokens, temperature, top_p, repetition_penalty (runtime/src/bin/serve.rs:1285-1292).
 
   python -m trapetum_amd run MODEL_DIR PROMPT.bin [--max-tokens 24] ...      one prompt, like gemma_run
+  python -m trapetum_amd run MODEL_DIR --prompt "text" ...                   with the folder's tokenizer.json
   python -m trapetum_amd generate MODEL_DIR --prompts-file ids.txt ...       many prompts, one id list per line
   python -m trapetum_amd replay --model DIR --dtype D --out DIR --max-tokens N   (same as bin/trace_run)
   python -m trapetum_amd random --config CONFIG.json --out DIR --seed S     write a random model folder
@@ -85,6 +86,8 @@ def main(argv=None):
     run.add_argument("model", nargs="?", help="folder with config.json and model.safetensors")
     run.add_argument("prompt", nargs="?", help="file of little-endian int32 token ids")
     run.add_argument("--prompt-ids", help="comma-separated token ids instead of a file")
+    run.add_argument("--prompt-text", "--prompt", dest="prompt_text", metavar="TEXT",
+                     help="a text prompt, encoded by the model folder's tokenizer.json (no special tokens added)")
     _add_sampling(run)
     gen = sub.add_parser("generate", help="generate for many prompts")
     gen.add_argument("model", nargs="?")
@@ -116,7 +119,19 @@ def main(argv=None):
         print(f"wrote {args.out}")
         return 0
     if args.command == "run":
-        if args.prompt_ids:
+        tok = None
+        if args.prompt_text is not None:
+            from .text import FolderTokenizer, TextError
+            if args.model is None:
+                ap.error("a text prompt needs a model folder with a tokenizer.json")
+            if args.prompt is not None:
+                ap.error("give a prompt file or --prompt, not both")
+            try:
+                tok = FolderTokenizer(args.model)
+                prompt = tok.encode(args.prompt_text)
+            except TextError as e:
+                raise SystemExit(str(e))
+        elif args.prompt_ids:
             prompt = [int(t) for t in args.prompt_ids.replace(",", " ").split()]
         elif args.prompt:
             prompt = _read_ids_bin(args.prompt)
@@ -124,6 +139,8 @@ def main(argv=None):
             ap.error("run needs a prompt file or --prompt-ids")
         out = _generate(args, [prompt])
         print("continuation ids:", out[0])
+        if tok is not None:
+            print("continuation text:", tok.decode(out[0]))
         return 0
     if args.command == "generate":
         with open(args.prompts_file) as f:
