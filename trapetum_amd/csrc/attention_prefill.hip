@@ -146,7 +146,11 @@ attn_prefill_k(PrefillArgs a) {
         if (PAGED && key < start) {
             int row = key;
             if (a.rows_cap > 0) {
+                // key % rows_cap without a division: a cached key lies less than window + 30 positions behind k_lo (the
+                // window's start rounded down to a tile), the window fits the ring and the ring has at least 16 rows,
+                // so the sum below is less than four rings: three conditional subtractions
                 row = ring_lo + (key - k_lo);
+                row = row >= a.rows_cap ? row - a.rows_cap : row;
                 row = row >= a.rows_cap ? row - a.rows_cap : row;
                 row = row >= a.rows_cap ? row - a.rows_cap : row;
             }
