@@ -441,12 +441,14 @@ rope_kv_write_vec_k(bf16_t* __restrict__ q, long q_stride, bf16_t* __restrict__ 
                     const int* __restrict__ row_seq, const int* __restrict__ row_pos,
                     const int* __restrict__ new_len, const int* __restrict__ table, int table_w,
                     bf16_t* __restrict__ k_pool, bf16_t* __restrict__ v_pool, int page, int rows_cap) {
-    __shared__ float cs[128], sn[128];
+    // cosine and sine of pair f at [f % 8][f / 8]: the threads of a wave, which turn neighbouring pieces of 8 pairs, then
+    // read neighbouring words (pair by pair in the pairs' own order, a wave's reads fell on four banks)
+    __shared__ float cs[8 * 16], sn[8 * 16];
     const int r = blockIdx.x, pos = row_pos[r], half = rot / 2;
     for (int f = threadIdx.x; f < half; f += 256) {
         const float ang = (float)pos * inv_freq[f];
-        cs[f] = cosf(ang);
-        sn[f] = sinf(ang);
+        cs[(f & 7) * 16 + (f >> 3)] = cosf(ang);
+        sn[(f & 7) * 16 + (f >> 3)] = sinf(ang);
     }
     size_t cache_at = 0;
     bool cached = false;
@@ -466,7 +468,7 @@ rope_kv_write_vec_k(bf16_t* __restrict__ q, long q_stride, bf16_t* __restrict__ 
     union Piece { uint4 u; bf16_t h[8]; };
     const int pieces = half / 8, heads = H + (k ? KV : 0);
     for (int item = threadIdx.x; item < heads * pieces; item += 256) {
-        const int j = item / pieces, f0 = (item - j * pieces) * 8;
+        const int j = item / pieces, piece = item - j * pieces, f0 = piece * 8;
         const bool is_q = j < H;
         bf16_t* x = is_q ? q + (size_t)r * q_stride + (size_t)j * hd : k + (size_t)r * k_stride + (size_t)(j - H) * hd;
         Piece lo, hi;
@@ -474,7 +476,7 @@ rope_kv_write_vec_k(bf16_t* __restrict__ q, long q_stride, bf16_t* __restrict__ 
         hi.u = *reinterpret_cast<const uint4*>(x + f0 + half);
 #pragma unroll
         for (int e = 0; e < 8; e++) {
-            const float x0 = bf16_to_f32(lo.h[e]), x1 = bf16_to_f32(hi.h[e]), c = cs[f0 + e], sv = sn[f0 + e];
+            const float x0 = bf16_to_f32(lo.h[e]), x1 = bf16_to_f32(hi.h[e]), c = cs[e * 16 + piece], sv = sn[e * 16 + piece];
             lo.h[e] = f32_to_bf16(x0 * c - x1 * sv);
             hi.h[e] = f32_to_bf16(x1 * c + x0 * sv);
         }
