@@ -302,7 +302,16 @@ static int add_rms_norm_launch(float* stream, const void* rows, int n_slices, lo
     else if (few && D > 1024 * 4 && D <= 640 * 8) TP_ADD_NORM_VEC(2, 640);
     else if (few && D > 640 * 8 && D <= 1024 * 8) TP_ADD_NORM_VEC(2, 1024);
     else if (vec && D <= 256 * 4) TP_ADD_NORM_VEC(1, 256);
+    // many rows: three chunks a lane and just the waves that fills (a width of 2,304 is 576 chunks: three waves a
+    // block, so that the CUs hold every block of 2,048 rows at once and no lane idles; 256 lanes left a quarter of
+    // them idle and the last quarter of the blocks waiting)
+    else if (vec && D <= 128 * 12) TP_ADD_NORM_VEC(3, 128);
+    else if (vec && D <= 192 * 12) TP_ADD_NORM_VEC(3, 192);
     else if (vec && D <= 256 * 12) TP_ADD_NORM_VEC(3, 256);
+    else if (vec && D <= 320 * 12) TP_ADD_NORM_VEC(3, 320);
+    else if (vec && D <= 384 * 12) TP_ADD_NORM_VEC(3, 384);
+    else if (vec && D <= 448 * 12) TP_ADD_NORM_VEC(3, 448);
+    else if (vec && D <= 512 * 12) TP_ADD_NORM_VEC(3, 512);
     else if (vec && D <= 512 * 16) TP_ADD_NORM_VEC(4, 512);
     else if (D <= 256 * 2) add_rms_norm_reg_k<TR, T, 2, 256><<<M, 256, 0, s>>>(stream, (const TR*)rows, n_slices, slice_stride, gp, ep, gn, en, (T*)out, D);
     else if (M <= 128 && D <= 1024 * 4) add_rms_norm_reg_k<TR, T, 4, 1024><<<M, 1024, 0, s>>>(stream, (const TR*)rows, n_slices, slice_stride, gp, ep, gn, en, (T*)out, D);
