@@ -393,8 +393,9 @@ static Plan plan_of(const GemmArgs& a) {
     if ((a.M <= 64 && !(a.M > 32 && a.N >= 32768)) || (a.M <= 256 && (long)tp_cdiv(a.M, 128) * tp_cdiv(a.N, 128) < 256)) {
         const long tiles = (long)tp_cdiv(a.M, 64) * tp_cdiv(a.N, 64);
         Tile t{2, 2};
-        // Up to 32 rows what such a product waits for is W, and a block that asks one k step ahead has 16 KB of it in
-        // flight: with two steps ahead (a second set of staging registers) the long loops gain, those of a gated product
+        // Up to 32 rows what such a product waits for is W: with a second set of staging registers, so that a step's
+        // loads are asked for a set earlier (the compiler still waits for all of them before a set's first use, so it
+        // is less than two whole steps in flight), the long loops gain, those of a gated product
         // (never sliced) and of the slices of 17 rows and more (2B gate/up at 16 rows 27.6 -> 23.0 us, 27B at 8 rows
         // 141 -> 126, 9B qkv at 32 rows 21.1 -> 18.1); slices of a few steps (up to 16 rows) and 64 rows do not.
         // A gated product with about a block a CU in these tiles gains more from 64 x 32 tiles, twice the blocks with
